@@ -111,4 +111,6 @@ def architecture_name(raw: dict[str, Any]) -> str:
     archs = raw.get("architectures")
     if isinstance(archs, list) and archs and isinstance(archs[0], str):
         return archs[0]
-    raise ConfigError("config.json has no 'architectures' list naming the model class")
+    if isinstance(raw.get("architecture"), str):       # the one-name spelling
+        return raw["architecture"]
+    raise ConfigError("config.json has no 'architectures' list (or 'architecture' name) naming the model class")

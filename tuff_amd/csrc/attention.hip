@@ -13,6 +13,10 @@
 //
 // Cache layout: K [page][kv_head][offset][hd], V [page][kv_head][hd][offset].
 //
+// Values may be of another width than keys (vd; V [page][kv_head][vd][offset]), and a head may
+// have a sink: a learned logit whose exponential counts once in the softmax's denominator and
+// that has neither key nor value (it is not scaled).
+//
 // This is the general kernel: any head size up to 256, any page size, float32 or
 // bfloat16 cache.  One wave per (token, head): lanes are keys for q.k, lanes are
 // channels for p.v.
@@ -26,7 +30,7 @@ template <typename T>
 __global__ __launch_bounds__(WAVE) void attention_general_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ req_of_token,
-    const int* __restrict__ positions, int H, int Hkv, int hd, int page_size, int window, float scale) {
+    const int* __restrict__ positions, int H, int Hkv, int hd, int vd, int page_size, int window, float scale, const float* __restrict__ sinks) {
     __shared__ float qs[MAX_PER_LANE * WAVE];
     __shared__ float ps[WAVE];
     __shared__ long long voff[WAVE];
@@ -51,9 +55,9 @@ __global__ __launch_bounds__(WAVE) void attention_general_kernel(
         long long base = 0;
         if (valid) {
             const long long page = table[kt / page_size];
-            const long long head_base = (page * Hkv + kvh) * page_size * (long long)hd;
-            base = head_base + (kt % page_size);          // V: [hd][page_size], this key's column
-            const T* krow = k_cache + head_base + (long long)(kt % page_size) * hd;
+            const long long head_base = (page * Hkv + kvh) * page_size;
+            base = head_base * vd + (kt % page_size);     // V: [vd][page_size], this key's column
+            const T* krow = k_cache + head_base * hd + (long long)(kt % page_size) * hd;
             float d = 0.f;
             for (int j = 0; j < hd; ++j) d = fmaf(qs[j], to_f32(krow[j]), d);
             s = d * scale;
@@ -77,34 +81,42 @@ __global__ __launch_bounds__(WAVE) void attention_general_kernel(
 #pragma unroll
             for (int i = 0; i < MAX_PER_LANE; ++i) {
                 const int j = lane + i * WAVE;
-                if (j < hd) acc[i] = fmaf(pj, to_f32(vcol[(long long)j * page_size]), acc[i]);
+                if (j < vd) acc[i] = fmaf(pj, to_f32(vcol[(long long)j * page_size]), acc[i]);
             }
         }
     }
-    T* o = out + ((long long)t * H + head) * hd;
-    const float inv = 1.0f / l;
+    T* o = out + ((long long)t * H + head) * vd;
+    float keep = 1.f;
+    if (sinks) {
+        // the sink joins the denominator under the common maximum
+        const float sk = sinks[head];
+        const float m_new = fmaxf(m, sk);
+        keep = expf(m - m_new);
+        l = l * keep + expf(sk - m_new);
+    }
+    const float inv = keep / l;
 #pragma unroll
     for (int i = 0; i < MAX_PER_LANE; ++i) {
         const int j = lane + i * WAVE;
-        if (j < hd) o[j] = from_f32<T>(acc[i] * inv);
+        if (j < vd) o[j] = from_f32<T>(acc[i] * inv);
     }
 }
 }  // namespace
 
 TUFF_EXPORT int tuff_attention_general(const void* q, const void* k_cache, const void* v_cache, void* out, int dt,
                                        const int* block_table, int max_blocks, const int* req_of_token,
-                                       const int* positions, int n_tokens, int H, int Hkv, int hd, int page_size,
-                                       int window, float scale, hipStream_t stream) {
+                                       const int* positions, int n_tokens, int H, int Hkv, int hd, int vd, int page_size,
+                                       int window, float scale, const float* sinks, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (hd > MAX_PER_LANE * WAVE || Hkv <= 0 || H % Hkv != 0) return -2;
+    if (hd > MAX_PER_LANE * WAVE || vd > MAX_PER_LANE * WAVE || vd <= 0 || Hkv <= 0 || H % Hkv != 0) return -2;
     dim3 grid(n_tokens, H), block(WAVE);
     if (dt == DT_F32)
         hipLaunchKernelGGL(attention_general_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_cache,
-                           (const float*)v_cache, (float*)out, block_table, max_blocks, req_of_token, positions, H, Hkv, hd,
-                           page_size, window, scale);
+                           (const float*)v_cache, (float*)out, block_table, max_blocks, req_of_token, positions, H, Hkv, hd, vd,
+                           page_size, window, scale, sinks);
     else
         hipLaunchKernelGGL(attention_general_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache,
-                           (const bf16_t*)v_cache, (bf16_t*)out, block_table, max_blocks, req_of_token, positions, H, Hkv, hd,
-                           page_size, window, scale);
+                           (const bf16_t*)v_cache, (bf16_t*)out, block_table, max_blocks, req_of_token, positions, H, Hkv, hd, vd,
+                           page_size, window, scale, sinks);
     return launch_status();
 }

@@ -36,6 +36,8 @@ MODULES = {
     "attention_mfma": "attention_mfma.hip",
     "attention_prefill": "attention_prefill.hip",
     "shortconv": "shortconv.hip",
+    "recurrent": "recurrent.hip",
+    "moe": "moe.hip",
     "sampling": "sampling.hip",
 }
 

@@ -188,3 +188,107 @@ TUFF_EXPORT int tuff_scatter_i32(int* dst, int n_dst, const int* src, int n_src,
     hipLaunchKernelGGL(scatter_i32_kernel, dim3(ceil_div(n, 256)), dim3(256), 0, stream, dst, n_dst, src, n_src, idx, n);
     return launch_status();
 }
+
+// ----------------------------------------------------------------- dynamic tanh
+// y_i = tanh(alpha x_i) w_i + b_i: a norm without statistics.  `rows` (optional) gathers input rows.
+template <typename TO>
+__global__ void dyt_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ b,
+                           const float* __restrict__ alpha, TO* __restrict__ out, const int* __restrict__ rows, int d) {
+    const int r = blockIdx.x;
+    const long long src = rows ? rows[r] : r;
+    const float a = alpha[0];
+    const float* xr = x + src * (long long)d;
+    TO* o = out + (long long)r * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<TO>(fmaf(tanhf(a * xr[i]), w[i], b[i]));
+}
+
+TUFF_EXPORT int tuff_dyt(const float* x, const float* w, const float* b, const float* alpha, void* out, int out_dt,
+                         const int* rows, int n_rows, int d, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    dim3 grid(n_rows), block(256);
+    if (out_dt == DT_F32) hipLaunchKernelGGL(dyt_kernel<float>, grid, block, 0, stream, x, w, b, alpha, (float*)out, rows, d);
+    else hipLaunchKernelGGL(dyt_kernel<bf16_t>, grid, block, 0, stream, x, w, b, alpha, (bf16_t*)out, rows, d);
+    return launch_status();
+}
+
+// ------------------------------------------------------------- activations
+// kind: 0 silu, 1 gelu (tanh form), 2 relu squared, 3 tanh, 4 sigmoid; evaluated in float32.
+__device__ __forceinline__ float activation(float z, int kind) {
+    switch (kind) {
+        case 0: return z / (1.0f + expf(-z));
+        case 1: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+        case 2: { const float r = fmaxf(z, 0.f); return r * r; }
+        case 3: return tanhf(z);
+        default: return 1.0f / (1.0f + expf(-z));
+    }
+}
+
+// act[t, f] = f(g) * u with g = gu[t, f], u = gu[t, F + f]: the gated product of a feed-forward whose
+// gate and up rows are stacked, for any of the activations above.
+template <typename T>
+__global__ void glu_kernel(const T* __restrict__ gu, T* __restrict__ act, long long n, int F, int kind) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long long t = i / F;
+    const int f = (int)(i - t * F);
+    act[i] = from_f32<T>(activation(to_f32(gu[t * 2 * F + f]), kind) * to_f32(gu[t * 2 * F + F + f]));
+}
+
+TUFF_EXPORT int tuff_glu(const void* gu, void* act, int dt, int n_tokens, int F, int kind, hipStream_t stream) {
+    const long long n = (long long)n_tokens * F;
+    if (n <= 0) return 0;
+    dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
+    if (dt == DT_F32) hipLaunchKernelGGL(glu_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)act, n, F, kind);
+    else hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)act, n, F, kind);
+    return launch_status();
+}
+
+// out[t, c] = f(in[t, c]) * (row_gate ? g(row_gate[t * gate_stride]) : 1): an activation, optionally times one
+// number a row (g: gate_kind, or -1 for the number as it is).  in and out may be the same memory.
+template <typename TI, typename TO>
+__global__ void act_rows_kernel(const TI* __restrict__ in, TO* __restrict__ out, long long n, int N, int kind,
+                                const float* __restrict__ row_gate, int gate_stride, int gate_kind) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = activation(to_f32(in[i]), kind);
+    if (row_gate) {
+        const float g = row_gate[(i / N) * gate_stride];
+        v *= gate_kind < 0 ? g : activation(g, gate_kind);
+    }
+    out[i] = from_f32<TO>(v);
+}
+
+TUFF_EXPORT int tuff_act_rows(const void* in, int in_dt, void* out, int out_dt, long long rows, int N, int kind,
+                              const float* row_gate, int gate_stride, int gate_kind, hipStream_t stream) {
+    const long long n = rows * N;
+    if (n <= 0) return 0;
+    dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
+#define LAUNCH(TI, TO) hipLaunchKernelGGL((act_rows_kernel<TI, TO>), grid, block, 0, stream, (const TI*)in, (TO*)out, n, N, kind, row_gate, gate_stride, gate_kind)
+    if (in_dt == DT_F32 && out_dt == DT_F32) LAUNCH(float, float);
+    else if (in_dt == DT_F32) LAUNCH(float, bf16_t);
+    else if (out_dt == DT_F32) LAUNCH(bf16_t, float);
+    else LAUNCH(bf16_t, bf16_t);
+#undef LAUNCH
+    return launch_status();
+}
+
+// ------------------------------------------------------------------ column padding
+// out[t, c] = c < N ? in[t, c] : 0 for c < Np: rows widened with zeros, for a product whose inner size
+// must be a multiple of the kernels' load width.
+template <typename T>
+__global__ void pad_cols_kernel(const T* __restrict__ in, T* __restrict__ out, long long n, int N, int Np) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long long t = i / Np;
+    const int c = (int)(i - t * Np);
+    out[i] = c < N ? in[t * N + c] : from_f32<T>(0.f);
+}
+
+TUFF_EXPORT int tuff_pad_cols(const void* in, void* out, int dt, long long rows, int N, int Np, hipStream_t stream) {
+    const long long n = rows * Np;
+    if (n <= 0) return 0;
+    dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
+    if (dt == DT_F32) hipLaunchKernelGGL(pad_cols_kernel<float>, grid, block, 0, stream, (const float*)in, (float*)out, n, N, Np);
+    else hipLaunchKernelGGL(pad_cols_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, n, N, Np);
+    return launch_status();
+}

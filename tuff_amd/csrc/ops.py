@@ -35,6 +35,28 @@ _SIGNATURES = {
         "tuff_cast": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_void_p],
         "tuff_fill_u32": [_c_void_p, ctypes.c_uint32, _c_ll, _c_void_p],
         "tuff_scatter_i32": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p],
+        "tuff_dyt": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tuff_glu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_act_rows": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tuff_pad_cols": [_c_void_p, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p],
+    },
+    "recurrent": {
+        "tuff_shift_mix": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                           _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_shift_state": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+        "tuff_conv_act": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_wkv_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_delta_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                            _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int,
+                                _c_float, _c_void_p],
+    },
+    "moe": {
+        "tuff_moe_route": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_moe_experts": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "gemm_f32": {
         "tuff_gemm_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -62,12 +84,12 @@ _SIGNATURES = {
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
         "tuff_rope_table": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_kv_write": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
-                          _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "attention": {
         "tuff_attention_general": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
-                                   _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                   _c_float, _c_void_p],
+                                   _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                   _c_float, _c_void_p, _c_void_p],
     },
     "attention_mfma": {
         "tuff_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -309,6 +331,55 @@ def scatter_i32(dst: torch.Tensor, src: torch.Tensor, idx: torch.Tensor) -> None
     _check(load("elementwise").tuff_scatter_i32(_gpu("dst", dst, torch.int32), dst.numel(), _gpu("src", src, torch.int32),
                                                 src.numel(), _gpu("idx", idx, torch.int32, (2 * n,)), n, _stream()),
            "scatter_i32")
+
+
+def dyt(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, alpha: torch.Tensor, out: torch.Tensor,
+        rows: Optional[torch.Tensor] = None) -> None:
+    """out = tanh(alpha * x[rows]) * w + b; x float32 [*, d], w and b float32 [d], alpha float32 [1]."""
+    n, d = out.shape
+    _gpu("x", x, torch.float32, (n if rows is None else None, d))
+    _check(load("elementwise").tuff_dyt(
+        x.data_ptr(), _gpu("w", w, torch.float32, (d,)), _gpu("b", b, torch.float32, (d,)),
+        _gpu("alpha", alpha, torch.float32, (1,)), _gpu("out", out), _dt(out),
+        _opt("rows", rows, torch.int32, (n,)), n, d, _stream()), "dyt")
+
+
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "relu2": 2, "tanh": 3, "sigmoid": 4}
+
+
+def glu(gu: torch.Tensor, act: torch.Tensor, activation: str) -> None:
+    """act[t, f] = activation(gu[t, f]) * gu[t, F + f]."""
+    n, F = act.shape
+    _check(load("elementwise").tuff_glu(
+        _gpu("gu", gu, act.dtype, (n, 2 * F)), _gpu("act", act), _dt(act), n, F, ACTIVATIONS[activation], _stream()), "glu")
+
+
+def act_rows(inp: torch.Tensor, out: torch.Tensor, activation: str, row_gate: Optional[torch.Tensor] = None,
+             gate_col: int = 0, gate_activation: Optional[str] = None) -> None:
+    """out = activation(inp), each row times gate_activation(row_gate[row, gate_col]) where row_gate
+    (float32 [rows, *]) is given (gate_activation None: the number as it is).  inp may be out."""
+    rows, N = out.shape
+    _gpu("inp", inp, shape=(rows, N))
+    _gpu("out", out)
+    gp, stride = None, 0
+    if row_gate is not None:
+        _gpu("row_gate", row_gate, torch.float32, (rows, None))
+        if not 0 <= gate_col < row_gate.shape[1]:
+            raise KernelError("act_rows: gate_col outside row_gate")
+        gp, stride = row_gate.data_ptr() + 4 * gate_col, row_gate.shape[1]
+    _check(load("elementwise").tuff_act_rows(
+        inp.data_ptr(), _dt(inp), out.data_ptr(), _dt(out), rows, N, ACTIVATIONS[activation], gp, stride,
+        -1 if gate_activation is None else ACTIVATIONS[gate_activation], _stream()), "act_rows")
+
+
+def pad_cols(inp: torch.Tensor, width: int) -> torch.Tensor:
+    """inp [rows, N] widened to [rows, width] with zeros."""
+    rows, N = inp.shape
+    if width < N:
+        raise KernelError("pad_cols: narrower than the input")
+    out = torch.empty(rows, width, dtype=inp.dtype, device=inp.device)
+    _check(load("elementwise").tuff_pad_cols(_gpu("inp", inp), out.data_ptr(), _dt(inp), rows, N, width, _stream()), "pad_cols")
+    return out
 
 
 # ------------------------------------------------------------------------------ GEMM
@@ -655,43 +726,50 @@ def rope_table(inv_freq: torch.Tensor, n_pos: int) -> torch.Tensor:
     return out
 
 
-def kv_write(k, v, k_cache, v_cache, slot_mapping, *, Hkv, hd, page_size) -> None:
+def kv_write(k, v, k_cache, v_cache, slot_mapping, *, Hkv, hd, page_size, vd=None) -> None:
+    """Rows of keys [T, Hkv * hd] and values [T, Hkv * vd] (vd: hd unless given) into the paged cache."""
     T = k.shape[0]
     dt = k.dtype
+    vd = hd if vd is None else int(vd)
     _gpu("k", k, shape=(T, Hkv * hd))
-    _gpu("v", v, dt, (T, Hkv * hd))
+    _gpu("v", v, dt, (T, Hkv * vd))
     P = k_cache.shape[0]
     _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
-    _gpu("v_cache", v_cache, dt, (P, Hkv, hd, page_size))
+    _gpu("v_cache", v_cache, dt, (P, Hkv, vd, page_size))
     _gpu("slot_mapping", slot_mapping, torch.int32, (T,))
     _check(load("rope_kv").tuff_kv_write(k.data_ptr(), v.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                                         _dt(k), slot_mapping.data_ptr(), T, Hkv, hd, page_size, _stream()),
+                                         _dt(k), slot_mapping.data_ptr(), T, Hkv, hd, vd, page_size, _stream()),
            "kv_write")
 
 
 # -------------------------------------------------------------------------- attention
 def attention_general(q, k_cache, v_cache, out, *, block_table, req_of_token, positions,
-                      H, Hkv, hd, page_size, window=0, scale=None) -> None:
+                      H, Hkv, hd, page_size, window=0, scale=None, vd=None, sinks=None) -> None:
+    """vd: width of a value where it is not the keys'.  sinks: float32 [H], a logit per head that counts
+    once in the softmax's denominator and has no value."""
     T = q.shape[0]
     dt = q.dtype
+    vd = hd if vd is None else int(vd)
     _gpu("q", q, shape=(T, H * hd))
-    _gpu("out", out, dt, (T, H * hd))
+    _gpu("out", out, dt, (T, H * vd))
     P = k_cache.shape[0]
     _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
-    _gpu("v_cache", v_cache, dt, (P, Hkv, hd, page_size))
+    _gpu("v_cache", v_cache, dt, (P, Hkv, vd, page_size))
+    _opt("sinks", sinks, torch.float32, (H,))
     _gpu("block_table", block_table, torch.int32)
     if block_table.dim() != 2:
         raise KernelError("attention: block_table must be [requests, blocks]")
     _gpu("req_of_token", req_of_token, torch.int32, (T,))
     _gpu("positions", positions, torch.int32, (T,))
-    if hd > 256 or H % Hkv:
-        raise KernelError(f"attention: head size {hd} / heads {H}:{Hkv} not supported")
+    if hd > 256 or vd > 256 or H % Hkv:
+        raise KernelError(f"attention: head size {hd} (values {vd}) / heads {H}:{Hkv} not supported")
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
     _check(load("attention").tuff_attention_general(
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q),
         block_table.data_ptr(), block_table.shape[1], req_of_token.data_ptr(), positions.data_ptr(),
-        T, H, Hkv, hd, page_size, int(window or 0), float(scale), _stream()), "attention_general")
+        T, H, Hkv, hd, vd, page_size, int(window or 0), float(scale), None if sinks is None else sinks.data_ptr(),
+        _stream()), "attention_general")
 
 
 ATTN_PARTITION = 256        # keys a partition of the matrix-core attention kernel covers
@@ -945,6 +1023,138 @@ def shortconv_state(bcx, state, *, q_start, q_len, state_slot, K) -> None:
     _check(load("shortconv").tuff_shortconv_state(
         bcx.data_ptr(), _dt(bcx), state.data_ptr(), q_start.data_ptr(), q_len.data_ptr(),
         state_slot.data_ptr(), R, d, K, _stream()), "shortconv_state")
+
+
+# -------------------------------------------------------------------- recurrent mixers
+def shift_mix(h, prev_state, mu, out, *, req_of_token, q_start, state_slot) -> None:
+    """out[s, t] = h[t] + (h[t - 1] - h[t]) * mu[s]; the row before a request's first token of the step is
+    prev_state[slot] (float32 [slots, d]).  h [T, d]; mu float32 [n, d]; out [n, T, d] of h's type."""
+    T, d = h.shape
+    n = mu.shape[0]
+    R = q_start.shape[0]
+    _check(load("recurrent").tuff_shift_mix(
+        _gpu("h", h), _dt(h), _gpu("prev_state", prev_state, torch.float32, (None, d)), _gpu("mu", mu, torch.float32, (n, d)),
+        _gpu("out", out, h.dtype, (n, T, d)), _gpu("req_of_token", req_of_token, torch.int32, (T,)),
+        _gpu("q_start", q_start, torch.int32, (R,)), _gpu("state_slot", state_slot, torch.int32, (R,)), T, d, n, _stream()),
+        "shift_mix")
+
+
+def shift_state(h, prev_state, *, q_start, q_len, state_slot) -> None:
+    """prev_state[slot] = the last row each request has in the step."""
+    T, d = h.shape
+    R = q_start.shape[0]
+    _check(load("recurrent").tuff_shift_state(
+        _gpu("h", h), _dt(h), _gpu("prev_state", prev_state, torch.float32, (None, d)),
+        _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
+        _gpu("state_slot", state_slot, torch.int32, (R,)), R, d, _stream()), "shift_state")
+
+
+CONV_ACT_MAX_TAPS = 17
+
+
+def conv_act(x, taps, state, out, *, req_of_token, q_start, state_slot, q_len=None, activation: Optional[str] = "silu") -> None:
+    """out[t, c] = activation(sum_j taps[c, j] x[t - (K - 1) + j, c]) along each request; rows before the
+    step's first come from state[slot] (float32 [slots, K - 1, C]; None with one tap).  With q_len the state
+    is then rewritten with the last K - 1 inputs; without, it is only read."""
+    T, C = x.shape
+    K = taps.shape[1]
+    R = q_start.shape[0]
+    if activation not in (None, "silu"):
+        raise KernelError("conv_act: activation is 'silu' or None")
+    if not 1 <= K <= CONV_ACT_MAX_TAPS:
+        raise KernelError(f"conv_act: 1 to {CONV_ACT_MAX_TAPS} taps, got {K}")
+    if K > 1:
+        _gpu("state", state, torch.float32, (None, K - 1, C))
+    _check(load("recurrent").tuff_conv_act(
+        _gpu("x", x), _dt(x), _gpu("taps", taps, torch.float32, (C, K)), None if K == 1 else state.data_ptr(),
+        _gpu("out", out, x.dtype, (T, C)), _gpu("req_of_token", req_of_token, torch.int32, (T,)),
+        _gpu("q_start", q_start, torch.int32, (R,)), _opt("q_len", q_len, torch.int32, (R,)),
+        _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, C, K, 1 if activation == "silu" else 0, _stream()), "conv_act")
+
+
+SCAN_MAX_DIM = 256
+
+
+def wkv_scan(r, k, v, lw, w0, u, state, out, *, q_start, q_len, state_slot, H, D) -> None:
+    """The decaying outer-product recurrence over each request's tokens of the step, from and to
+    state[slot] (float32 [slots, H, D, D]): o = (S + diag(u) k v^T)^T r, then S = diag(w) S + k v^T with
+    w = exp(-exp(lw + w0)).  r, k, v [T, H * D]; lw float32 [T, H * D]; w0 float32 [H * D]; u float32 [H, D];
+    out float32 [T, H * D]."""
+    T = r.shape[0]
+    R = q_start.shape[0]
+    dt = r.dtype
+    if D > SCAN_MAX_DIM:
+        raise KernelError(f"wkv_scan: head size {D} above {SCAN_MAX_DIM}")
+    _check(load("recurrent").tuff_wkv_scan(
+        _gpu("r", r, shape=(T, H * D)), _gpu("k", k, dt, (T, H * D)), _gpu("v", v, dt, (T, H * D)), _dt(r),
+        _gpu("lw", lw, torch.float32, (T, H * D)), _gpu("w0", w0, torch.float32, (H * D,)), _gpu("u", u, torch.float32, (H, D)),
+        _gpu("state", state, torch.float32, (None, H, D, D)), _gpu("out", out, torch.float32, (T, H * D)),
+        _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
+        _gpu("state_slot", state_slot, torch.int32, (R,)), R, H, D, _stream()), "wkv_scan")
+
+
+def delta_scan(q, k, v, a, dt_bias, A_log, b, state, out, *, q_start, q_len, state_slot, H, Hk, D, Dv) -> None:
+    """The gated delta rule over each request's tokens of the step, from and to state[slot] (float32
+    [slots, H, D, Dv]): S = g S; e = beta (v - S^T k); S = S + k e^T; o = S^T q, with q and k made unit
+    vectors per head (q also times D^-1/2), g = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b).
+    q, k [T, Hk * D]; v [T, H * Dv]; a float32 [T, H * D]; b float32 [T, H]; out float32 [T, H * Dv]."""
+    T = q.shape[0]
+    R = q_start.shape[0]
+    dt = q.dtype
+    if D > SCAN_MAX_DIM or Hk < 1 or H % Hk:
+        raise KernelError(f"delta_scan: key size {D} (at most {SCAN_MAX_DIM}) / heads {H}:{Hk} not supported")
+    _check(load("recurrent").tuff_delta_scan(
+        _gpu("q", q, shape=(T, Hk * D)), _gpu("k", k, dt, (T, Hk * D)), _gpu("v", v, dt, (T, H * Dv)), _dt(q),
+        _gpu("a", a, torch.float32, (T, H * D)), _gpu("dt_bias", dt_bias, torch.float32, (H * D,)),
+        _gpu("A_log", A_log, torch.float32, (H,)), _gpu("b", b, torch.float32, (T, H)),
+        _gpu("state", state, torch.float32, (None, H, D, Dv)), _gpu("out", out, torch.float32, (T, H * Dv)),
+        _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
+        _gpu("state_slot", state_slot, torch.int32, (R,)), R, H, Hk, D, Dv, _stream()), "delta_scan")
+
+
+def head_norm_gate(o, w, gate, out, *, H, Dv, eps, per_head_weight: bool, gate_activation: Optional[str]) -> None:
+    """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * w * f(gate[t, h]); o float32 [T, H * Dv]; w float32
+    [H * Dv] (per_head_weight) or [Dv] (shared by the heads); gate and out [T, H * Dv] of the compute type."""
+    T = o.shape[0]
+    _check(load("recurrent").tuff_head_norm_gate(
+        _gpu("o", o, torch.float32, (T, H * Dv)), _gpu("w", w, torch.float32, (H * Dv if per_head_weight else Dv,)),
+        Dv if per_head_weight else 0, _gpu("gate", gate, out.dtype, (T, H * Dv)), _dt(out),
+        {None: 0, "silu": 1, "sigmoid": 2}[gate_activation], _gpu("out", out, shape=(T, H * Dv)), T, H, Dv, float(eps), _stream()),
+        "head_norm_gate")
+
+
+# ------------------------------------------------------------------ mixture of experts
+def moe_route(z, ids, wts, *, E, top, weights: str = "sigmoid") -> None:
+    """ids, wts [T, top]: the `top` largest of z[t, :E] (float32 [T, >= E]; the lower index wins a tie) and
+    their weights, sigmoid(z) each on its own or a softmax over the chosen."""
+    T = z.shape[0]
+    _gpu("z", z, torch.float32)
+    if z.dim() != 2 or z.shape[1] < E:
+        raise KernelError("moe_route: z must be [tokens, >= experts]")
+    _check(load("moe").tuff_moe_route(z.data_ptr(), z.shape[1], _gpu("ids", ids, torch.int32, (T, top)),
+                                      _gpu("wts", wts, torch.float32, (T, top)), T, E, top,
+                                      {"sigmoid": 0, "softmax": 1}[weights], _stream()), "moe_route")
+
+
+def moe_experts(h, w_up, w_down, ids, wts, residual, *, activation: str = "relu2", scale_input: bool = True) -> None:
+    """residual[t] += sum over the token's choices of W_down[e] act(W_up[e] x), x = h[t] times the choice's
+    weight (scale_input) or the product times it.  h [T, d]; w_up [E, F, d]; w_down [E, d, F], all of one type."""
+    T, d = h.shape
+    E, F, _ = w_up.shape
+    top = ids.shape[1]
+    dt = h.dtype
+    _gpu("h", h)
+    _gpu("w_up", w_up, dt, (E, F, d))
+    _gpu("w_down", w_down, dt, (E, d, F))
+    _gpu("ids", ids, torch.int32, (T, top))
+    _gpu("wts", wts, torch.float32, (T, top))
+    _gpu("residual", residual, torch.float32, (T, d))
+    a = torch.empty(T * top, F, dtype=dt, device=h.device)
+    y = torch.empty(T * top, d, dtype=torch.float32, device=h.device)
+    _check(load("moe").tuff_moe_experts(h.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), _dt(h), ids.data_ptr(),
+                                        wts.data_ptr(), a.data_ptr(), y.data_ptr(), residual.data_ptr(), T, d, F, top,
+                                        {"relu2": 0, "silu": 1, "gelu_tanh": 2}[activation], int(scale_input), _stream()),
+           "moe_experts")
 
 
 # --------------------------------------------------------------------------- sampling

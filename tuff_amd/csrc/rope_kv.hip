@@ -291,17 +291,15 @@ __global__ void rope_table_kernel(const float* __restrict__ inv_freq, int n_freq
 template <typename T>
 __global__ __launch_bounds__(WAVE) void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v,
                                                         T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                                        const int* __restrict__ slot_mapping, int Hkv, int hd, int page_size) {
+                                                        const int* __restrict__ slot_mapping, int Hkv, int hd, int vd, int page_size) {
     const int t = blockIdx.x, kvh = blockIdx.y;
     const long long slot = slot_mapping[t];
     if (slot < 0) return;
     const long long page = slot / page_size, off = slot % page_size;
-    const long long head_base = (page * Hkv + kvh) * page_size * hd;
-    const long long src = ((long long)t * Hkv + kvh) * hd;
-    for (int j = threadIdx.x; j < hd; j += WAVE) {
-        k_cache[head_base + off * hd + j] = k[src + j];
-        v_cache[head_base + (long long)j * page_size + off] = v[src + j];
-    }
+    const long long head_base = (page * Hkv + kvh) * page_size;
+    const long long ksrc = ((long long)t * Hkv + kvh) * hd, vsrc = ((long long)t * Hkv + kvh) * vd;
+    for (int j = threadIdx.x; j < hd; j += WAVE) k_cache[head_base * hd + off * hd + j] = k[ksrc + j];
+    for (int j = threadIdx.x; j < vd; j += WAVE) v_cache[head_base * vd + (long long)j * page_size + off] = v[vsrc + j];
 }
 }  // namespace
 
@@ -363,12 +361,12 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
 }
 
 TUFF_EXPORT int tuff_kv_write(const void* k, const void* v, void* k_cache, void* v_cache, int dt,
-                              const int* slot_mapping, int n_tokens, int Hkv, int hd, int page_size,
+                              const int* slot_mapping, int n_tokens, int Hkv, int hd, int vd, int page_size,
                               hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     dim3 grid(n_tokens, Hkv), block(WAVE);
-    if (dt == DT_F32) hipLaunchKernelGGL(kv_write_kernel<float>, grid, block, 0, stream, (const float*)k, (const float*)v, (float*)k_cache, (float*)v_cache, slot_mapping, Hkv, hd, page_size);
-    else hipLaunchKernelGGL(kv_write_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping, Hkv, hd, page_size);
+    if (dt == DT_F32) hipLaunchKernelGGL(kv_write_kernel<float>, grid, block, 0, stream, (const float*)k, (const float*)v, (float*)k_cache, (float*)v_cache, slot_mapping, Hkv, hd, vd, page_size);
+    else hipLaunchKernelGGL(kv_write_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)k_cache, (bf16_t*)v_cache, slot_mapping, Hkv, hd, vd, page_size);
     return launch_status();
 }
 

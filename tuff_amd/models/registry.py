@@ -45,7 +45,19 @@ def config_from_dict(raw: dict) -> ModelConfig:
 
 
 def load_config(model_dir: str) -> ModelConfig:
-    return config_from_dict(read_config_json(model_dir))
+    """The folder's configuration.  A configuration that leaves sizes to the tensors' shapes (it has a
+    with_shapes method) is completed from the checkpoint's headers; no tensor is read for it."""
+    cfg = config_from_dict(read_config_json(model_dir))
+    if hasattr(cfg, "with_shapes"):
+        from ..weights.loader import Checkpoint
+        from ..weights.safetensors_io import SafetensorsError
+        try:
+            ck = Checkpoint(model_dir)
+        except (SafetensorsError, OSError):
+            return cfg                    # no readable checkpoint: the loader says so when the weights are asked for
+        names = set(ck.names())
+        cfg = cfg.with_shapes(lambda n: ck.shape(n) if n in names else None)
+    return cfg
 
 
 def build_model(cfg: ModelConfig):
@@ -56,6 +68,9 @@ def _register_builtin() -> None:
     from ..config.lfm2 import Lfm2Config
     from .lfm2 import build_lfm2
     register_architecture(Lfm2Config.architecture, Lfm2Config, build_lfm2)
+    from ..config.pafodra import PafodraConfig
+    from .pafodra import build_pafodra
+    register_architecture(PafodraConfig.architecture, PafodraConfig, build_pafodra)
 
 
 _register_builtin()

@@ -28,22 +28,32 @@ class AttentionMixer(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
                  names: dict[str, str], qk_norm_eps: Optional[float] = None,
                  position: Optional[PositionEncoding] = None, window: Optional[int] = None,
-                 scale: Optional[float] = None, aliases: Optional[dict[str, tuple]] = None):
-        """names: checkpoint names of 'q', 'k', 'v', 'o' and, with qk_norm_eps, 'q_norm', 'k_norm'."""
+                 scale: Optional[float] = None, aliases: Optional[dict[str, tuple]] = None,
+                 value_dim: Optional[int] = None):
+        """names: checkpoint names of 'q', 'k', 'v', 'o' and, with qk_norm_eps, 'q_norm', 'k_norm'; with a
+        'sink' among them the heads have sinks.  value_dim: width of a value head (default: head_dim)."""
         if num_heads % num_kv_heads:
             raise ValueError(f"heads {num_heads} must be a multiple of kv heads {num_kv_heads}")
         if head_dim > 256:
             raise ValueError(f"head size {head_dim} above 256 is not supported by the attention kernels")
         self.d, self.H, self.Hkv, self.hd = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.vd = self.hd if value_dim is None else int(value_dim)
+        if self.vd > 256 or self.vd < 1:
+            raise ValueError(f"value size {self.vd} is outside 1..256")
+        if self.vd != self.hd and (qk_norm_eps is not None or position is not None):
+            raise ValueError("values of another width than keys go with plain queries and keys only (no per-head "
+                             "norm, no position encoding)")
+        self.has_sink = "sink" in names
+        self.sinks = None
         self.eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.position, self.window = position, (int(window) if window else None)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.hd)
         self.names = dict(names)
         al = aliases or {}
         self.qkv = Linear([names["q"], names["k"], names["v"]], self.d,
-                          [self.H * self.hd, self.Hkv * self.hd, self.Hkv * self.hd],
+                          [self.H * self.hd, self.Hkv * self.hd, self.Hkv * self.vd],
                           aliases=[al.get("q", ()), al.get("k", ()), al.get("v", ())])
-        self.out = Linear(names["o"], self.H * self.hd, self.d, aliases=[al.get("o", ())])
+        self.out = Linear(names["o"], self.H * self.vd, self.d, aliases=[al.get("o", ())])
         self._al = al
         self.q_norm_w = self.k_norm_w = None
 
@@ -62,6 +72,8 @@ class AttentionMixer(Mixer):
                       WeightDecl(self.names["k_norm"], (self.hd,), "norm", aliases=self._al.get("k_norm", ()))]
         if self.position is not None:
             decls += self.position.weight_decls()
+        if self.has_sink:
+            decls.append(WeightDecl(self.names["sink"], (self.H,), "normal", aliases=self._al.get("sink", ())))
         return decls
 
     def kernel_modules(self):
@@ -74,7 +86,7 @@ class AttentionMixer(Mixer):
         return self.position.token_inputs() if self.position is not None else []
 
     def cache_spec(self):
-        return PagedKV(self.Hkv, self.hd, self.window)
+        return PagedKV(self.Hkv, self.hd, self.window, value_dim=None if self.vd == self.hd else self.vd)
 
     def bind(self, weights, rt: Runtime):
         self.rt = rt
@@ -88,25 +100,35 @@ class AttentionMixer(Mixer):
                 self.k_norm_w = self.k_norm_w.float()
         if self.position is not None:
             self.position.bind(weights, rt)
+        if self.has_sink:
+            self.sinks = weights[self.names["sink"]].float().contiguous()
 
     def forward(self, h, ctx, cache, residual, write_cache: bool = True, next_norm=None) -> None:
         T = h.shape[0]
-        H, Hkv, hd = self.H, self.Hkv, self.hd
+        H, Hkv, hd, vd = self.H, self.Hkv, self.hd, self.vd
         qkv = self.qkv.forward(h)
-        q = self.rt.empty(T, H * hd)
-        o = self.rt.empty(T, H * hd)
+        q = self.rt.empty(T, H * hd) if vd == hd else None
+        o = self.rt.empty(T, H * vd)
         norm = dict(eps=self.eps or 0.0, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w)
         tables = self.position.rotary_tables() if self.position is not None else None
         fused = self.position is None or tables is not None
         # a position encoding of its own: norm, then its apply(), then the cache write
         k = None if fused else self.rt.empty(T, Hkv * hd)
 
-        one_kernel = (fused and tables is not None and ctx.max_q_len == 1 and ops.attention_decode_fused_supported(
+        one_kernel = (fused and tables is not None and ctx.max_q_len == 1 and self.sinks is None and ops.attention_decode_fused_supported(
             qkv.dtype, H, Hkv, hd, cache.page_size, tables[1], tables[2]))
 
         def over_the_cache(ctx):
             """What depends on where the step's tokens lie: positions, cache slots, block tables."""
             g = ctx.groups[cache.group]
+            if vd != hd:
+                # keys and values of different widths: the rows are cut out and written as they are
+                qq = qkv[:, :H * hd].contiguous()
+                if write_cache:
+                    ops.kv_write(qkv[:, H * hd:(H + Hkv) * hd].contiguous(), qkv[:, (H + Hkv) * hd:].contiguous(),
+                                 cache.k, cache.v, g.slot_mapping, Hkv=Hkv, hd=hd, vd=vd, page_size=cache.page_size)
+                self.attend(qq, o, ctx, cache, g)
+                return
             if one_kernel:
                 # single tokens, heads of 64: norm, rotation, cache write and attention in one kernel
                 ops.attention_decode_fused(qkv, cache.k, cache.v, o, block_table=g.block_table, req_info=ctx.req_info,
@@ -178,7 +200,7 @@ class AttentionMixer(Mixer):
 
     def attend(self, q, o, ctx, cache, g) -> None:
         G = self.H // self.Hkv
-        if ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
+        if self.vd == self.hd and self.sinks is None and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
             common = dict(block_table=g.block_table, req_info=ctx.req_info, H=self.H, Hkv=self.Hkv, hd=self.hd,
                           page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
                           scale=self.scale)
@@ -204,4 +226,4 @@ class AttentionMixer(Mixer):
         ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
                               req_of_token=ctx.req_of_token, positions=ctx.positions,
                               H=self.H, Hkv=self.Hkv, hd=self.hd, page_size=cache.page_size,
-                              window=self.window or 0, scale=self.scale)
+                              window=self.window or 0, scale=self.scale, vd=self.vd, sinks=self.sinks)

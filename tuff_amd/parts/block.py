@@ -3,6 +3,9 @@
 PreNormBlock is the reference's layer (src/lfm25_engine.c:370-419):
     x += mixer(norm1(x));  x += ffn(norm2(x))
 with the residual stream x in float32.  A feed-forward of None leaves out the second half.
+
+ParallelBlock has one norm whose output both sublayers read:
+    h = norm(x);  x += mixer(h) + ffn(h)
 """
 from __future__ import annotations
 
@@ -84,3 +87,45 @@ class PreNormBlock(Block):
         if consumer.accepts_pending_norm and hasattr(norm, "pending"):
             return norm.pending(x)
         return norm.forward(x)
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(Block):
+    """x <- x + mixer(h) + ffn(h) with h = norm(x): mixer and feed-forward read the same normed rows and
+    both add into the float32 stream.  ffn None: the mixer alone."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, ffn: Optional[FeedForward] = None):
+        self.norm, self.mixer, self.ffn = norm, mixer, ffn
+
+    def _parts(self):
+        return [p for p in (self.norm, self.mixer, self.ffn) if p is not None]
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self._parts())
+
+    @property
+    def records_portions(self):
+        return all(p.records_portions for p in self._parts())
+
+    def weight_decls(self):
+        return [d for p in self._parts() for d in p.weight_decls()]
+
+    def kernel_modules(self):
+        return [m for p in self._parts() for m in p.kernel_modules()]
+
+    def token_inputs(self):
+        return [t for p in self._parts() for t in p.token_inputs()]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        for p in self._parts():
+            p.bind(weights, rt)
+
+    def forward(self, x, ctx, cache, write_cache: bool = True) -> None:
+        h = self.norm.forward(x)            # computed before either sublayer touches x
+        kw = {"next_norm": None} if self.mixer.adds_once_through_linear else {}
+        self.mixer.forward(h, ctx, cache, x, write_cache, **kw)
+        if self.ffn is not None:
+            kw = {"next_norm": None} if self.ffn.adds_once_through_linear else {}
+            self.ffn.forward(h, ctx, x, **kw)

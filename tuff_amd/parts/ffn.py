@@ -1,4 +1,9 @@
-"""SwiGLU feed-forward: W_down (silu(W_gate h) * (W_up h)), silu(g) = g / (1 + exp(-g)).
+"""Feed-forwards.
+
+GatedMLP: W_down (act(W_gate h + b_g) * (W_up h + b_u)) + b_d with act silu or the tanh form of gelu, biases optional.
+MoE: routed experts W_down act(W_up x) chosen per token by a router, and an optional shared expert.
+
+SwiGLU feed-forward: W_down (silu(W_gate h) * (W_up h)), silu(g) = g / (1 + exp(-g)).
 Reference: src/lfm25_gpu.cu:583-618 (gate and up in one pass with the activation fused),
 src/lfm25_engine.c:412-419.  Gate and up are one product; with bfloat16 weights their rows are
 interleaved and the activation is the product's epilogue.
@@ -8,7 +13,7 @@ from __future__ import annotations
 import torch
 
 from ..csrc import ops
-from .base import FEED_FORWARDS, FeedForward, Runtime
+from .base import FEED_FORWARDS, FeedForward, Runtime, WeightDecl
 from .linear import Linear
 
 
@@ -65,3 +70,144 @@ class SwiGLU(FeedForward):
             act = self.rt.empty(h.shape[0], self.width, dtype=gu.dtype)
             ops.swiglu(gu, act)
         self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
+
+
+@FEED_FORWARDS.register("gated")
+class GatedMLP(FeedForward):
+    """W_down (act(W_gate h + b_gate) * (W_up h + b_up)) + b_down.  activation: "silu" or "gelu_tanh"
+    (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))).  names: 'gate', 'up' [F, d], 'down' [d, F] and, with
+    bias=True, 'gate.b', 'up.b' [F], 'down.b' [d]."""
+    graph_safe = True
+    records_portions = True
+    adds_once_through_linear = True
+
+    def __init__(self, hidden_size: int, ffn_dim: int, *, names: dict[str, str], activation: str = "gelu_tanh",
+                 bias: bool = False):
+        if activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"unknown activation '{activation}'")
+        self.d, self.F, self.activation, self.has_bias = int(hidden_size), int(ffn_dim), activation, bool(bias)
+        self._names = dict(names)
+        self._make(self.F)
+        self._decls = self.gate_up.weight_decls() + self.down.weight_decls()
+
+    def _make(self, width: int) -> None:
+        n = self._names
+        self.gate_up = Linear([n["gate"], n["up"]], self.d, [width, width],
+                              bias=[n["gate.b"], n["up.b"]] if self.has_bias else None)
+        self.down = Linear(n["down"], width, self.d, bias=n["down.b"] if self.has_bias else None)
+        self.width = width
+
+    def weight_decls(self):
+        return self._decls
+
+    def kernel_modules(self):
+        return ["elementwise"]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        n = self._names
+        g, u, dn = (weights[n[k]] for k in ("gate", "up", "down"))
+        if self.F % 8 and all(t.dtype == torch.bfloat16 for t in (g, u, dn)):
+            # zero rows of gate and up (with zero biases: act(0) * 0 = 0) and zero columns of down: the same function
+            pad = -self.F % 8
+            weights = dict(weights)
+            weights[n["gate"]] = torch.cat([g, g.new_zeros(pad, self.d)])
+            weights[n["up"]] = torch.cat([u, u.new_zeros(pad, self.d)])
+            weights[n["down"]] = torch.cat([dn, dn.new_zeros(self.d, pad)], dim=1).contiguous()
+            if self.has_bias:
+                for k in ("gate.b", "up.b"):
+                    weights[n[k]] = torch.cat([weights[n[k]], weights[n[k]].new_zeros(pad)])
+            self._make(self.F + pad)
+        self.gate_up.bind(weights, rt)
+        self.down.bind(weights, rt)
+
+    def forward(self, h, ctx, residual, next_norm=None) -> None:
+        gu = self.gate_up.forward(h)
+        act = self.rt.empty(h.shape[0], self.width, dtype=gu.dtype)
+        ops.glu(gu, act, self.activation)
+        self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
+
+
+@FEED_FORWARDS.register("moe")
+class MoE(FeedForward):
+    """Routed experts, each W_down act(W_up x) without biases, and an optional shared expert of the same form.
+
+    Router logits z = W_router h are float32 products.  The `top` largest are chosen per token (the lower
+    index wins a tie).  router_weights "sigmoid": a choice's weight is sigmoid(z), each on its own; "softmax":
+    a softmax over the chosen.  scale_input: the weight multiplies the expert's input (sum_e expert_e(w_e h));
+    else its output.  The shared expert runs for every token and is multiplied by sigmoid(W_sg h), one number a
+    token (names['shared.sg'], [1, d]); without that name it is added as it is.
+    names: 'router' [E, d]; 'experts': a list of (up [F, d], down [d, F]) names; optional 'shared.up',
+    'shared.down', 'shared.sg'."""
+    graph_safe = True
+    records_portions = True
+
+    def __init__(self, hidden_size: int, num_experts: int, top: int, expert_dim: int, *, names: dict,
+                 activation: str = "relu2", router_weights: str = "sigmoid", scale_input: bool = True,
+                 shared_dim: int = 0):
+        self.d, self.E, self.top, self.F = int(hidden_size), int(num_experts), int(top), int(expert_dim)
+        if not 1 <= self.top <= self.E:
+            raise ValueError(f"top {self.top} of {self.E} experts")
+        if activation not in ("relu2", "silu", "gelu_tanh"):
+            raise ValueError(f"unknown activation '{activation}'")
+        self.activation, self.router_weights, self.scale_input = activation, router_weights, bool(scale_input)
+        self.names = dict(names)
+        if len(self.names["experts"]) != self.E:
+            raise ValueError("one (up, down) pair of names per expert")
+        self.Fs = int(shared_dim)
+        self.shared_gate = self.Fs > 0 and "shared.sg" in self.names
+        rows = [self.names["router"]] + ([self.names["shared.sg"]] if self.shared_gate else [])
+        self.router = Linear(rows, self.d, [self.E] + ([1] if self.shared_gate else []), float32=True)
+        self.shared_up = self.shared_down = None
+        if self.Fs:
+            self._make_shared(self.Fs)
+
+    def _make_shared(self, width: int) -> None:
+        self.shared_up = Linear(self.names["shared.up"], self.d, width)
+        self.shared_down = Linear(self.names["shared.down"], width, self.d)
+
+    def weight_decls(self):
+        decls = self.router.weight_decls()
+        for up, down in self.names["experts"]:
+            decls += [WeightDecl(up, (self.F, self.d), "normal", role="projection"),
+                      WeightDecl(down, (self.d, self.F), "normal", role="projection")]
+        if self.Fs:
+            decls += [WeightDecl(self.names["shared.up"], (self.Fs, self.d), "normal", role="projection"),
+                      WeightDecl(self.names["shared.down"], (self.d, self.Fs), "normal", role="projection")]
+        return decls
+
+    def kernel_modules(self):
+        return ["moe", "elementwise", "gemm_f32"]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        self.router.bind(weights, rt)
+        self.w_up = torch.stack([weights[up] for up, _ in self.names["experts"]]).contiguous()           # [E, F, d]
+        self.w_down = torch.stack([weights[down] for _, down in self.names["experts"]]).contiguous()     # [E, d, F]
+        if self.Fs:
+            up, down = weights[self.names["shared.up"]], weights[self.names["shared.down"]]
+            if self.Fs % 8 and up.dtype == torch.bfloat16 and down.dtype == torch.bfloat16:
+                pad = -self.Fs % 8
+                weights = dict(weights)
+                weights[self.names["shared.up"]] = torch.cat([up, up.new_zeros(pad, self.d)])
+                weights[self.names["shared.down"]] = torch.cat([down, down.new_zeros(self.d, pad)], dim=1).contiguous()
+                self._make_shared(self.Fs + pad)
+            self.shared_up.bind(weights, rt)
+            self.shared_down.bind(weights, rt)
+
+    def forward(self, h, ctx, residual) -> None:
+        T = h.shape[0]
+        z = self.router.forward(h, out_dtype=torch.float32)                  # [T, E (+ 1)]
+        ids = torch.empty(T, self.top, dtype=torch.int32, device=h.device)
+        wts = torch.empty(T, self.top, dtype=torch.float32, device=h.device)
+        ops.moe_route(z, ids, wts, E=self.E, top=self.top, weights=self.router_weights)
+        ops.moe_experts(h, self.w_up, self.w_down, ids, wts, residual, activation=self.activation,
+                        scale_input=self.scale_input)
+        if self.Fs:
+            a = self.shared_up.forward(h)
+            # the gate is one number a token and the second product is linear: it goes onto the activations
+            if self.shared_gate:
+                ops.act_rows(a, a, self.activation, row_gate=z, gate_col=self.E, gate_activation="sigmoid")
+            else:
+                ops.act_rows(a, a, self.activation)
+            self.shared_down.forward(a, accumulate_into=residual)

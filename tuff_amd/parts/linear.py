@@ -15,14 +15,18 @@ from .base import Runtime, WeightDecl
 class Linear:
     def __init__(self, names: Sequence[str] | str, in_features: int,
                  out_features: Sequence[int] | int, aliases: Sequence[Sequence[str]] | None = None,
-                 swiglu_pair: bool = False, bias: Sequence[str] | str | None = None):
+                 swiglu_pair: bool = False, bias: Sequence[str] | str | None = None, float32: bool = False):
         """swiglu_pair: the two stacked tensors are the gate and the up matrix of a SwiGLU; with
         bfloat16 weights their rows are interleaved so that forward(..., swiglu=True) can apply
         silu(gate) * up in the product's epilogue.
         bias: checkpoint names of a bias vector per stacked tensor ([out] each), y = x W^T + b.  The
         products' epilogues have no bias: it is added by a kernel of its own after the product, and a
         projection with one takes none of the fused ways (activation, convolution or the next norm in
-        the product's epilogue); the result is the same function."""
+        the product's epilogue); the result is the same function.
+        float32: the weight is kept in float32 and the product runs in true float32 whatever the run's
+        type (a router, whose logits decide which experts a token takes).
+        An input size that is no multiple of 8 (the bfloat16 kernels read 16 bytes at a time) is filled up
+        with zero columns when the weight is bound, and forward() widens its input with zeros: the same sums."""
         self.names = [names] if isinstance(names, str) else list(names)
         outs = [out_features] if isinstance(out_features, int) else list(out_features)
         if len(outs) != len(self.names):
@@ -40,6 +44,8 @@ class Linear:
         if self.bias_names is not None and len(self.bias_names) != len(self.names):
             raise ValueError("one bias per stacked tensor")
         self.bias = None              # bound: float32 [out]
+        self.float32 = bool(float32)
+        self.k_padded = self.in_features     # bound: the inner size the kernels see
 
     def weight_decls(self) -> list[WeightDecl]:
         decls = [WeightDecl(n, (o, self.in_features), "normal", aliases=a, role="projection")
@@ -51,6 +57,8 @@ class Linear:
     def bind(self, weights: dict[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
         ws = [weights[n] for n in self.names]
+        if self.float32:
+            ws = [w.to(torch.float32) for w in ws]
         if len(ws) == 1:
             self.weight = ws[0]
         else:
@@ -63,8 +71,10 @@ class Linear:
                 self.weight = torch.cat(ws, dim=0).contiguous()
         if self.weight.dtype == torch.bfloat16:
             if self.in_features % 8 != 0:
-                raise ValueError(f"{self.names[0]}: the bfloat16 matrix kernels need an input size that is a "
-                                 f"multiple of 8, got {self.in_features}")
+                self.k_padded = -(-self.in_features // 8) * 8
+                wide = self.weight.new_zeros(self.out_features, self.k_padded)
+                wide[:, :self.in_features] = self.weight
+                self.weight = wide
             self.weight = ops.tile_weight(self.weight)       # the order the kernels stream it in
         if self.bias_names is not None:
             self.bias = torch.cat([weights[n].to(torch.float32).reshape(-1) for n in self.bias_names]).contiguous()
@@ -135,6 +145,8 @@ class Linear:
                 x, pending = pending.tensor(), None
         if pending is None:
             T = x.shape[0]
+            if self.k_padded != self.in_features and x.shape[1] == self.in_features:
+                x = ops.pad_cols(x, self.k_padded)
             if x.dtype != w.dtype:
                 # a weight stored in 32-bit stays so: run this product in float32
                 if w.dtype != torch.float32:
@@ -159,7 +171,7 @@ class Linear:
             layout = None
             if (nxt is not None and pending is None and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16
                     and self.in_features % 8 == 0):
-                layout = ops.gemm_emit_layout(T, self.out_features, self.in_features)
+                layout = ops.gemm_emit_layout(T, self.out_features, self.k_padded)
             if layout is not None:
                 # the norm that follows reads the sum just made: leave it its operand and row sums
                 xw = torch.empty(T, self.out_features, dtype=torch.bfloat16, device=dev)

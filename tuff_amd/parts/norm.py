@@ -1,4 +1,8 @@
-"""RMSNorm: y = x / sqrt(mean(x^2) + eps) * w, in float32 (src/lfm25_gpu.cu:235,244)."""
+"""Norms of the residual stream, in float32.
+
+RMSNorm: y = x / sqrt(mean(x^2) + eps) * w (src/lfm25_gpu.cu:235,244).
+DynamicTanh: y = tanh(alpha x) w + b with a learned scalar alpha; no mean, no variance.
+"""
 from __future__ import annotations
 
 from typing import Optional
@@ -77,4 +81,35 @@ class RMSNorm(Norm):
         n = x.shape[0] if rows is None else rows.shape[0]
         out = self.rt.empty(n, self.dim)
         ops.rmsnorm(x, self.weight, out, self.eps, rows)
+        return out
+
+
+@NORMS.register("dyt")
+class DynamicTanh(Norm):
+    """y = tanh(alpha * x) * w + b: an element-wise squashing in place of a norm; it reads no statistics of
+    the row, so it has no eps.  names: checkpoint names of 'weight' [d], 'bias' [d] and 'alpha' (a scalar)."""
+    graph_safe = True
+    records_portions = True
+
+    def __init__(self, dim: int, *, names: dict[str, str]):
+        self.dim, self.names = int(dim), dict(names)
+
+    def weight_decls(self):
+        return [WeightDecl(self.names["weight"], (self.dim,), "norm"),
+                WeightDecl(self.names["bias"], (self.dim,), "normal"),
+                WeightDecl(self.names["alpha"], (), "norm", alt_shapes=((1,),))]
+
+    def kernel_modules(self):
+        return ["elementwise"]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        self.weight_f32 = weights[self.names["weight"]].float().contiguous()
+        self.bias_f32 = weights[self.names["bias"]].float().contiguous()
+        self.alpha_f32 = weights[self.names["alpha"]].float().reshape(1).contiguous()
+
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        n = x.shape[0] if rows is None else rows.shape[0]
+        out = self.rt.empty(n, self.dim)
+        ops.dyt(x, self.weight_f32, self.bias_f32, self.alpha_f32, out, rows)
         return out
