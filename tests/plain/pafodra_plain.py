@@ -150,12 +150,20 @@ def expert(x, up, down, rnd=_same):
     return rnd(torch.relu(x @ up.T) ** 2) @ down.T
 
 
-def moe_ff(n, W, spec, rnd=_same):
+def moe_ff(n, W, spec, rnd=_same, margins: list | None = None):
     """Sigmoid scores, the `top` largest chosen, their scores (not renormalised) multiply the
-    experts' inputs; a shared expert for every token, gated by one sigmoid per token."""
+    experts' inputs; a shared expert for every token, gated by one sigmoid per token.
+    margins: gets, per token, how far the last chosen logit lies above the first one left out, in units of
+    the logits' spread (infinite where every expert is chosen): a small one is a close call, which rounding
+    may decide the other way."""
     T, d = n.shape
     E, top = spec["router"]["experts"], spec["router"]["top"]
-    s = torch.sigmoid(n @ W["router"].T)
+    z = n @ W["router"].T
+    s = torch.sigmoid(z)
+    if margins is not None:
+        zs = torch.sort(z, dim=-1, descending=True).values
+        gap = (zs[:, top - 1] - zs[:, top]) if top < E else torch.full((T,), math.inf, dtype=z.dtype)
+        margins.append(gap / z.pow(2).mean().sqrt())
     order = torch.sort(s, dim=-1, descending=True, stable=True).indices[:, :top]
     out = torch.zeros(T, d, dtype=n.dtype)
     for t in range(T):
@@ -172,9 +180,10 @@ def sub(weights: dict, prefix: str) -> dict:
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
 
-def forward(cfg: dict, weights: dict, tokens, rnd=_same, layers_out: list | None = None) -> torch.Tensor:
+def forward(cfg: dict, weights: dict, tokens, rnd=_same, layers_out: list | None = None,
+            margins_out: list | None = None) -> torch.Tensor:
     """Logits [T, vocab] of one sequence from its start.  layers_out: gets the residual stream after
-    every layer run."""
+    every layer run.  margins_out: gets the routers' margins [T] of every layer run with experts (moe_ff)."""
     W = {k: v.to(F64) for k, v in weights.items()}
     eps = cfg["norm"]["eps"]
     x = W["embed"][torch.as_tensor(tokens, dtype=torch.long)] * cfg["embedding"]["scale"]
@@ -194,7 +203,7 @@ def forward(cfg: dict, weights: dict, tokens, rnd=_same, layers_out: list | None
         spec = layer.get("mlp")
         if spec is not None:
             fw = sub(W, p + "mlp.")
-            y = y + (dense_ff(n, fw, rnd) if spec["kind"] == "dense" else moe_ff(n, fw, spec, rnd))
+            y = y + (dense_ff(n, fw, rnd) if spec["kind"] == "dense" else moe_ff(n, fw, spec, rnd, margins_out))
         x = x + y
         if layers_out is not None:
             layers_out.append(x.clone())

@@ -560,9 +560,12 @@ constexpr int COMBINE_MAX_PARTS = 2048;
 template <int PER, int BATCH>
 __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                               bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                                              int H, int hd, int window, int n_parts, int part_keys) {
+                                                              int H, int hd, int window, int n_parts, int part_keys,
+                                                              const float* __restrict__ sinks) {
     const long long row = blockIdx.x;                      // token * H + head
     const int lane = threadIdx.x;
+    // a head's sink: a logit without key or value that counts once in the denominator (none: -inf, which adds 0)
+    const float sink = sinks ? sinks[row % H] : -INFINITY;
     float m_l = -INFINITY, l_l = 0.f;
     if (lane < n_parts) {                                  // read before the position is known: rows exist for all partitions
         const float* ml = ws_ml + (row * n_parts + lane) * 2;
@@ -573,7 +576,7 @@ __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __res
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
     const int p_lo = lo / part_keys, p_hi = pos / part_keys;
     const bool valid = lane >= p_lo && lane <= p_hi && l_l > 0.f;
-    const float M = wave_max(valid ? m_l : -INFINITY);
+    const float M = fmaxf(wave_max(valid ? m_l : -INFINITY), sink);
     const float w_l = valid ? __expf(m_l - M) : 0.f;
     const float wl_l = w_l * (valid ? l_l : 0.f);
     const float* o = ws_o + row * n_parts * hd;
@@ -602,6 +605,7 @@ __global__ __launch_bounds__(WAVE) void attn_combine64_kernel(const float* __res
             }
         }
     }
+    if (sinks) L += __expf(sink - M);
     const float inv = 1.0f / L;
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
@@ -620,7 +624,8 @@ constexpr int COMBINE_MAX_GROUPS = COMBINE_MAX_PARTS / COMBINE_GROUP;
 
 __global__ __launch_bounds__(COMBINE_WAVES * WAVE) void attn_combine_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
                                                                             bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                                                            int H, int hd, int window, int n_parts, int part_keys) {
+                                                                            int H, int hd, int window, int n_parts, int part_keys,
+                                                                            const float* __restrict__ sinks) {
     __shared__ float wts[COMBINE_MAX_PARTS], wls[COMBINE_MAX_PARTS];
     __shared__ float grp_acc[COMBINE_MAX_GROUPS][256], grp_l[COMBINE_MAX_GROUPS];
     __shared__ float red[COMBINE_WAVES];
@@ -637,6 +642,8 @@ __global__ __launch_bounds__(COMBINE_WAVES * WAVE) void attn_combine_kernel(cons
     __syncthreads();
 #pragma unroll
     for (int w = 0; w < COMBINE_WAVES; ++w) M = fmaxf(M, red[w]);
+    const float sink = sinks ? sinks[row % H] : -INFINITY;
+    M = fmaxf(M, sink);
     for (int p = p_lo + tid; p <= p_hi; p += COMBINE_WAVES * WAVE) {
         const float l = ml[p * 2 + 1];
         const float w = l > 0.f ? __expf(ml[p * 2] - M) : 0.f;
@@ -691,6 +698,7 @@ __global__ __launch_bounds__(COMBINE_WAVES * WAVE) void attn_combine_kernel(cons
                 if (d < hd) acc[j] += grp_acc[grp][d];
             }
         }
+        if (sinks) L += __expf(sink - M);
         const float inv = 1.0f / L;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -747,18 +755,18 @@ void launch_partition(dim3 grid, hipStream_t stream, const bf16_t* q, bf16_t* kc
 // Merges, for every (token, head) of n_tokens tokens, the partial results of its partitions of
 // part_keys keys each.
 static int launch_merge(const float* ws_o, const float* ws_ml, bf16_t* out, const int* positions, int n_tokens, int H, int hd,
-                 int window, int n_parts, int part_keys, hipStream_t stream) {
+                 int window, int n_parts, int part_keys, hipStream_t stream, const float* sinks = nullptr) {
     const dim3 grid((unsigned)((long long)n_tokens * H));
     if (n_parts <= WAVE) {
 #define COMBINE(PER, BATCH) hipLaunchKernelGGL((attn_combine64_kernel<PER, BATCH>), grid, dim3(WAVE), 0, stream, ws_o, ws_ml, out, \
-                                               positions, H, hd, window, n_parts, part_keys)
+                                               positions, H, hd, window, n_parts, part_keys, sinks)
         if (hd <= 64) { if (n_parts <= 8) COMBINE(1, 8); else if (n_parts <= 16) COMBINE(1, 16); else COMBINE(1, 32); }
         else if (hd <= 128) { if (n_parts <= 8) COMBINE(2, 8); else COMBINE(2, 16); }
         else COMBINE(4, 8);
 #undef COMBINE
     } else {
         hipLaunchKernelGGL(attn_combine_kernel, grid, dim3(COMBINE_WAVES * WAVE), 0, stream, ws_o, ws_ml, out, positions, H, hd,
-                           window, n_parts, part_keys);
+                           window, n_parts, part_keys, sinks);
     }
     return launch_status();
 }
@@ -774,7 +782,7 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
                             float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
                             const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
                             int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
-                            int n_parts, hipStream_t stream) {
+                            int n_parts, hipStream_t stream, const float* sinks = nullptr) {
     if (n_tokens <= 0 || n_qblocks <= 0) return 0;
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0 || n_parts < 1) return -2;
     if (Hkv > 65535 || n_qblocks > 65535 || n_parts > COMBINE_MAX_PARTS) return -2;
@@ -795,7 +803,7 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
     int rc = launch_status();
     if (rc) return rc;
     return launch_merge((const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, n_tokens, H, hd, window, n_parts, PART,
-                        stream);
+                        stream, sinks);
 }
 
 // The number of lanes of a wave that fetch page numbers for partition `part` with pages of page_size
@@ -838,6 +846,17 @@ TUFF_EXPORT int tuff_attention_mfma(const void* q, const void* k_cache, const vo
                             positions, n_tokens, H, Hkv, hd, page_size, window, scale, n_parts, stream);
 }
 
+// The same with a sink per head (sinks float32 [H], or null): a logit that has neither key nor value and
+// counts once, unscaled, in the softmax's denominator.  It enters where a row's partitions are merged.
+TUFF_EXPORT int tuff_attention_mfma_sinks(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                          float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
+                                          const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
+                                          int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
+                                          int n_parts, const float* sinks, hipStream_t stream) {
+    return launch_attention(q, k_cache, v_cache, out, ws_o, ws_ml, block_table, max_blocks, blk, n_qblocks, nb, req_info,
+                            positions, n_tokens, H, Hkv, hd, page_size, window, scale, n_parts, stream, sinks);
+}
+
 // A step of single tokens (request r's token is row r) over heads of 64 channels, from the projected
 // rows qkv [n_tokens, (H + 2 Hkv) * 64]: per-head RMSNorm of q and k (weights [64] of type norm_dt, or
 // null), half-split rotation over the whole head by inv_freq [32] (angles [n_angles][2][32]: the
@@ -876,6 +895,15 @@ TUFF_EXPORT int tuff_attention_merge(const float* ws_o, const float* ws_ml, void
     if (n_tokens <= 0) return 0;
     if (hd > 256 || n_parts < 1 || n_parts > COMBINE_MAX_PARTS || part_keys < 1) return -2;
     return launch_merge(ws_o, ws_ml, (bf16_t*)out, positions, n_tokens, H, hd, window, n_parts, part_keys, stream);
+}
+
+// The same with a sink per head (sinks float32 [H], or null): exp(sink) joins every row's denominator.
+TUFF_EXPORT int tuff_attention_merge_sinks(const float* ws_o, const float* ws_ml, void* out, const int* positions, int n_tokens,
+                                           int H, int hd, int window, int n_parts, int part_keys, const float* sinks,
+                                           hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (hd > 256 || n_parts < 1 || n_parts > COMBINE_MAX_PARTS || part_keys < 1) return -2;
+    return launch_merge(ws_o, ws_ml, (bf16_t*)out, positions, n_tokens, H, hd, window, n_parts, part_keys, stream, sinks);
 }
 
 // ------------------------------------------------- the same attention without an allocation

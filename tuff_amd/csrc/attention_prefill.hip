@@ -48,7 +48,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     bf16_t* __restrict__ out, const int* __restrict__ block_table, int max_blocks,
     const int2* __restrict__ blk, const int4* __restrict__ req_info,
     int H, int Hkv, int hd, int page_size, int window, float scale_log2e,
-    int seg_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml) {
+    int seg_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml, const float* __restrict__ sinks) {
     constexpr int KC = HDP / 32;          // 32-wide chunks of the head dimension
     constexpr int DB = HDP / 16;          // 16-wide blocks of output channels
     constexpr int HC = HDP / 8;           // 16-byte chunks of a K row
@@ -397,7 +397,14 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             }
             continue;
         }
-        const float inv = 1.0f / l;
+        float inv = 1.0f / l;
+        if (sinks) {
+            // the head's sink joins the denominator under the common reference exponent (base 2 here)
+            const float s2 = sinks[qrow[nb] % H] * 1.4426950408889634f;
+            const float m_all = fmaxf(m_run[nb], s2);
+            const float keep = __builtin_amdgcn_exp2f(m_run[nb] - m_all);
+            inv = keep / (l * keep + __builtin_amdgcn_exp2f(s2 - m_all));
+        }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
             const int dim = db * 16 + 4 * g;
@@ -413,7 +420,8 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
 template <int HDP, int NBW, int AHEAD>
 int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, bf16_t* out,
            const int* bt, int max_blocks, const int2* blk, const int4* req_info,
-           int H, int Hkv, int hd, int ps, int window, float scale_log2e, int seg_keys, float* ws_o, float* ws_ml) {
+           int H, int Hkv, int hd, int ps, int window, float scale_log2e, int seg_keys, float* ws_o, float* ws_ml,
+           const float* sinks) {
     auto kern = attn_prefill_kernel<HDP, NBW, AHEAD>;
     constexpr int lds = 2 * (STEP * (HDP + 8) + HDP * VROW) * 2;
     static bool set = false;
@@ -422,7 +430,7 @@ int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, con
         set = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(NT), lds, stream, q, kc, vc, out, bt, max_blocks, blk, req_info,
-                       H, Hkv, hd, ps, window, scale_log2e, seg_keys, ws_o, ws_ml);
+                       H, Hkv, hd, ps, window, scale_log2e, seg_keys, ws_o, ws_ml, sinks);
     return launch_status();
 }
 }  // namespace
@@ -438,11 +446,13 @@ TUFF_EXPORT int tuff_attention_prefill_block_columns(int hd) { return hd <= 128 
 // the partial results go to ws_o [tokens * H * n_segs * hd] and ws_ml [tokens * H * n_segs * 2] in the
 // layout of the single-token kernel's partitions, to be merged by tuff_attention_merge with
 // part_keys = seg_keys.
-TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                       const int* block_table, int max_blocks, const int* blk, int n_qblocks,
-                                       const int* req_info, int H, int Hkv, int hd, int page_size, int window,
-                                       float scale, int n_segs, int seg_keys, float* ws_o, float* ws_ml,
-                                       hipStream_t stream) {
+// sinks (float32 [H], or null): a logit per head that counts once, unscaled, in the denominator and has no
+// value; with key segments it enters at the merge instead (tuff_attention_merge_sinks), not here.
+TUFF_EXPORT int tuff_attention_prefill_sinks(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                             const int* block_table, int max_blocks, const int* blk, int n_qblocks,
+                                             const int* req_info, int H, int Hkv, int hd, int page_size, int window,
+                                             float scale, int n_segs, int seg_keys, float* ws_o, float* ws_ml,
+                                             const float* sinks, hipStream_t stream) {
     if (n_qblocks <= 0) return 0;
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0) return -2;
     if (Hkv > 65535 || !(scale > 0.f)) return -2;
@@ -456,11 +466,20 @@ TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const
     dim3 grid(n_qblocks * Hkv, 1, n_segs);
     const float sl = scale * 1.4426950408889634f;
 #define GO(HDP, NBW, AHEAD) return launch<HDP, NBW, AHEAD>(grid, stream, Q, K, V, (bf16_t*)out, block_table, max_blocks, (const int2*)blk, \
-                                             (const int4*)req_info, H, Hkv, hd, page_size, window, sl, seg_keys, ws_o, ws_ml)
+                                             (const int4*)req_info, H, Hkv, hd, page_size, window, sl, seg_keys, ws_o, ws_ml, n_segs > 1 ? nullptr : sinks)
     if (hd <= 32) GO(32, 2, 3);
     else if (hd <= 64) GO(64, 2, 2);
     else if (hd <= 96) GO(96, 2, 2);
     else if (hd <= 128) GO(128, 2, 2);
     else GO(256, 1, 1);
 #undef GO
+}
+
+TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       const int* block_table, int max_blocks, const int* blk, int n_qblocks,
+                                       const int* req_info, int H, int Hkv, int hd, int page_size, int window,
+                                       float scale, int n_segs, int seg_keys, float* ws_o, float* ws_ml,
+                                       hipStream_t stream) {
+    return tuff_attention_prefill_sinks(q, k_cache, v_cache, out, block_table, max_blocks, blk, n_qblocks, req_info, H, Hkv, hd,
+                                        page_size, window, scale, n_segs, seg_keys, ws_o, ws_ml, nullptr, stream);
 }

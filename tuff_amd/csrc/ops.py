@@ -36,7 +36,7 @@ _SIGNATURES = {
         "tuff_fill_u32": [_c_void_p, ctypes.c_uint32, _c_ll, _c_void_p],
         "tuff_scatter_i32": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p],
         "tuff_dyt": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
-        "tuff_glu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_glu": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_act_rows": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
         "tuff_pad_cols": [_c_void_p, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p],
     },
@@ -50,7 +50,7 @@ _SIGNATURES = {
                           _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_delta_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                             _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
-        "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int,
+        "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int,
                                 _c_float, _c_void_p],
     },
     "moe": {
@@ -95,6 +95,11 @@ _SIGNATURES = {
         "tuff_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                                 _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
+        "tuff_attention_mfma_sinks": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                                      _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
+                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p],
+        "tuff_attention_merge_sinks": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                       _c_void_p, _c_void_p],
         "tuff_attention_merge": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_void_p],
         "tuff_attention_decode_fused": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -109,6 +114,9 @@ _SIGNATURES = {
         "tuff_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
                                    _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                                    _c_void_p, _c_void_p, _c_void_p],
+        "tuff_attention_prefill_sinks": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
+                                         _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
+                                         _c_void_p, _c_void_p, _c_void_p, _c_void_p],
         "tuff_attention_prefill_block_columns": [_c_int],
     },
     "shortconv": {
@@ -348,10 +356,10 @@ ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "relu2": 2, "tanh": 3, "sigmoid": 4}
 
 
 def glu(gu: torch.Tensor, act: torch.Tensor, activation: str) -> None:
-    """act[t, f] = activation(gu[t, f]) * gu[t, F + f]."""
+    """act[t, f] = activation(gu[t, f]) * gu[t, F + f]; gu of act's type or float32."""
     n, F = act.shape
     _check(load("elementwise").tuff_glu(
-        _gpu("gu", gu, act.dtype, (n, 2 * F)), _gpu("act", act), _dt(act), n, F, ACTIVATIONS[activation], _stream()), "glu")
+        _gpu("gu", gu, shape=(n, 2 * F)), _dt(gu), _gpu("act", act), _dt(act), n, F, ACTIVATIONS[activation], _stream()), "glu")
 
 
 def act_rows(inp: torch.Tensor, out: torch.Tensor, activation: str, row_gate: Optional[torch.Tensor] = None,
@@ -780,12 +788,14 @@ def attention_mfma_supported(dtype, hd: int, page_size: int) -> bool:
 
 
 def attention_mfma(q, k_cache, v_cache, out, *, block_table, blocks, nb, req_info, positions,
-                   H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None) -> None:
+                   H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None, sinks=None) -> None:
     """Matrix-core attention over the paged bfloat16 cache.  blocks: int32 [n_blocks, 2] from
     query_blocks(), or None when every request's columns fit one block (block b = request b).
     req_info: int32 [R, 4] = (first token in the step, tokens, first position, -) per request.
-    max_ctx_len bounds every position + 1 of the step."""
+    max_ctx_len bounds every position + 1 of the step.  sinks: float32 [H] or None, a logit per head that
+    counts once in the softmax's denominator and has no value."""
     T = q.shape[0]
+    _opt("sinks", sinks, torch.float32, (H,))
     if not attention_mfma_supported(q.dtype, hd, page_size):
         raise KernelError(f"attention_mfma: needs bfloat16, a head size that is a multiple of 8 (got {hd}) "
                           f"and a page size that is a multiple of 16 (got {page_size})")
@@ -817,11 +827,13 @@ def attention_mfma(q, k_cache, v_cache, out, *, block_table, blocks, nb, req_inf
         scale = 1.0 / math.sqrt(hd)
     ws_o = torch.empty(T * H * n_parts * hd, dtype=torch.float32, device=q.device)
     ws_ml = torch.empty(T * H * n_parts * 2, dtype=torch.float32, device=q.device)
-    _check(load("attention_mfma").tuff_attention_mfma(
-        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), ws_o.data_ptr(), ws_ml.data_ptr(),
-        block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk, nb,
-        req_info.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, page_size,
-        int(window or 0), float(scale), n_parts, _stream()), "attention_mfma")
+    args = (q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), ws_o.data_ptr(), ws_ml.data_ptr(),
+            block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk, nb,
+            req_info.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, page_size, int(window or 0), float(scale), n_parts)
+    if sinks is None:
+        _check(load("attention_mfma").tuff_attention_mfma(*args, _stream()), "attention_mfma")
+    else:
+        _check(load("attention_mfma").tuff_attention_mfma_sinks(*args, sinks.data_ptr(), _stream()), "attention_mfma")
 
 
 def attention_decode_fused_supported(dtype, H: int, Hkv: int, hd: int, page_size: int, rotary_dim: int, interleaved: bool) -> bool:
@@ -891,7 +903,7 @@ PREFILL_MIN_SEGMENT = 1024       # keys; shorter segments are not worth their me
 
 
 def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info,
-                      H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None, positions=None) -> None:
+                      H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None, positions=None, sinks=None) -> None:
     """Matrix-core attention for steps with prompt portions: a workgroup walks over all keys of a
     block of query columns, keys and values staged through LDS; writes `out` directly.
     blocks: int32 [n_blocks, 2] from query_blocks(q_len, G, attention_prefill_block_columns(hd) // 16),
@@ -901,6 +913,7 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
     segments' results as a step of single tokens merges its partitions.  Then every row of `out` is
     written, also those of tokens no block covers (with meaningless values)."""
     T = q.shape[0]
+    _opt("sinks", sinks, torch.float32, (H,))      # a logit per head that counts once in the denominator and has no value
     if not attention_mfma_supported(q.dtype, hd, page_size):
         raise KernelError(f"attention_prefill: needs bfloat16, a head size that is a multiple of 8 (got {hd}) "
                           f"and a page size that is a multiple of 16 (got {page_size})")
@@ -941,15 +954,16 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
         ws_ml = torch.empty(T * H * n_segs * 2, dtype=torch.float32, device=q.device)
     else:
         n_segs, seg_keys = 1, 0
-    _check(load("attention_prefill").tuff_attention_prefill(
+    _check(load("attention_prefill").tuff_attention_prefill_sinks(
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
         block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk,
         req_info.data_ptr(), H, Hkv, hd, page_size, int(window or 0), float(scale), n_segs, seg_keys,
-        None if ws_o is None else ws_o.data_ptr(), None if ws_ml is None else ws_ml.data_ptr(), _stream()), "attention_prefill")
+        None if ws_o is None else ws_o.data_ptr(), None if ws_ml is None else ws_ml.data_ptr(),
+        None if sinks is None else sinks.data_ptr(), _stream()), "attention_prefill")
     if n_segs > 1:
-        _check(load("attention_mfma").tuff_attention_merge(ws_o.data_ptr(), ws_ml.data_ptr(), out.data_ptr(), positions.data_ptr(),
-                                                           T, H, hd, int(window or 0), n_segs, seg_keys, _stream()),
-               "attention_merge")
+        _check(load("attention_mfma").tuff_attention_merge_sinks(
+            ws_o.data_ptr(), ws_ml.data_ptr(), out.data_ptr(), positions.data_ptr(), T, H, hd, int(window or 0), n_segs, seg_keys,
+            None if sinks is None else sinks.data_ptr(), _stream()), "attention_merge")
 
 
 def query_blocks(q_len, G: int, nb: int, ctx_len=None):
@@ -1114,11 +1128,12 @@ def delta_scan(q, k, v, a, dt_bias, A_log, b, state, out, *, q_start, q_len, sta
 
 def head_norm_gate(o, w, gate, out, *, H, Dv, eps, per_head_weight: bool, gate_activation: Optional[str]) -> None:
     """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * w * f(gate[t, h]); o float32 [T, H * Dv]; w float32
-    [H * Dv] (per_head_weight) or [Dv] (shared by the heads); gate and out [T, H * Dv] of the compute type."""
+    [H * Dv] (per_head_weight) or [Dv] (shared by the heads); out [T, H * Dv] of the compute type, gate of that
+    type or float32."""
     T = o.shape[0]
     _check(load("recurrent").tuff_head_norm_gate(
         _gpu("o", o, torch.float32, (T, H * Dv)), _gpu("w", w, torch.float32, (H * Dv if per_head_weight else Dv,)),
-        Dv if per_head_weight else 0, _gpu("gate", gate, out.dtype, (T, H * Dv)), _dt(out),
+        Dv if per_head_weight else 0, _gpu("gate", gate, shape=(T, H * Dv)), _dt(gate), _dt(out),
         {None: 0, "silu": 1, "sigmoid": 2}[gate_activation], _gpu("out", out, shape=(T, H * Dv)), T, H, Dv, float(eps), _stream()),
         "head_norm_gate")
 

@@ -261,9 +261,9 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
 // ---------------------------------------------------------- per-head unit norm, weight and gate
 // y[t][h][j] = o[t][h][j] / sqrt(mean_j o^2 + eps) * w[(h * w_stride) + j] * f(gate[t][h][j]);
 // f: 0 identity, 1 silu, 2 sigmoid.  A wave per (token, head).
-template <typename T>
+template <typename TG, typename T>
 __global__ __launch_bounds__(WAVE) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w, int w_stride,
-                                                              const T* __restrict__ gate, int gate_fn, T* __restrict__ y,
+                                                              const TG* __restrict__ gate, int gate_fn, T* __restrict__ y,
                                                               int H, int Dv, float eps) {
     const long long row = (long long)blockIdx.x * H + blockIdx.y;
     const float* src = o + row * Dv;
@@ -357,11 +357,14 @@ TUFF_EXPORT int tuff_delta_scan(const void* q, const void* k, const void* v, int
     return dt == DT_F32 ? launch_scan<float, true>(p, n_requests, stream) : launch_scan<bf16_t, true>(p, n_requests, stream);
 }
 
-TUFF_EXPORT int tuff_head_norm_gate(const float* o, const float* w, int w_stride, const void* gate, int dt, int gate_fn,
+// gate_dt: type of the gate's rows (float32 sums of a product may come in as they are); dt: type of y.
+TUFF_EXPORT int tuff_head_norm_gate(const float* o, const float* w, int w_stride, const void* gate, int gate_dt, int dt, int gate_fn,
                                     void* y, int n_tokens, int H, int Dv, float eps, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     dim3 grid(n_tokens, H), block(WAVE);
-    if (dt == DT_F32) hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, block, 0, stream, o, w, w_stride, (const float*)gate, gate_fn, (float*)y, H, Dv, eps);
-    else hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, block, 0, stream, o, w, w_stride, (const bf16_t*)gate, gate_fn, (bf16_t*)y, H, Dv, eps);
+    if (dt == DT_F32 && gate_dt == DT_F32) hipLaunchKernelGGL((head_norm_gate_kernel<float, float>), grid, block, 0, stream, o, w, w_stride, (const float*)gate, gate_fn, (float*)y, H, Dv, eps);
+    else if (gate_dt == DT_F32) hipLaunchKernelGGL((head_norm_gate_kernel<float, bf16_t>), grid, block, 0, stream, o, w, w_stride, (const float*)gate, gate_fn, (bf16_t*)y, H, Dv, eps);
+    else if (dt == DT_BF16) hipLaunchKernelGGL((head_norm_gate_kernel<bf16_t, bf16_t>), grid, block, 0, stream, o, w, w_stride, (const bf16_t*)gate, gate_fn, (bf16_t*)y, H, Dv, eps);
+    else return -2;
     return launch_status();
 }

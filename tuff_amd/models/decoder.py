@@ -33,12 +33,15 @@ class DecoderModel:
                  blocks: list[Block], final_norm: Norm, head: Optional[WeightDecl] = None,
                  schedule: Optional[list[LayerRun]] = None, max_positions: Optional[int] = None,
                  eos_token_id: Optional[int] = None, embedding_scale: float = 1.0,
-                 logit_scale: float = 1.0, logit_softcap: Optional[float] = None):
+                 logit_scale: float = 1.0, logit_softcap: Optional[float] = None, pad_hidden: bool = False):
         """head=None: the head is the embedding (tied), as the reference does when the file has
         no output matrix (src/lfm25_model.c:128-131).
         embedding_scale: the embedding rows are multiplied by it on their way into the residual stream.
         logit_scale, logit_softcap: logits = head(norm(x)) * logit_scale, then, with a cap c,
-        c * tanh(logits / c).  The reference has none of the three (scale 1, no cap), which are the defaults."""
+        c * tanh(logits / c).  The reference has none of the three (scale 1, no cap), which are the defaults.
+        pad_hidden: a hidden size that is no multiple of 8 is served in bfloat16 too, by zero columns (for a
+        model all of whose parts take such a size); without it such a model is refused when it is bound."""
+        self.pad_hidden = bool(pad_hidden)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.embedding_decl, self.head_decl = embedding, head
         self.blocks, self.final_norm = list(blocks), final_norm
@@ -139,12 +142,20 @@ class DecoderModel:
         self._head_cast: Optional[torch.Tensor] = None
         if self.head.dtype != rt.dtype and self.head.dtype != torch.float32:
             raise TypeError(f"head weight of type {self.head.dtype} in a {rt.dtype} run")
+        self._head_k = self.hidden_size
         if self.head.dtype == torch.bfloat16:
             # the matrix kernels stream a tile-major copy; a tied embedding keeps its rows for the lookup
-            if self.hidden_size % 8 != 0:
+            head = self.head
+            if self.hidden_size % 8 != 0 and not self.pad_hidden:
                 raise ValueError(f"the bfloat16 matrix kernels need a hidden size that is a multiple of 8, "
                                  f"got {self.hidden_size}")
-            self.head = ops.tile_weight(self.head)
+            if self.hidden_size % 8 != 0:
+                # the kernels read 16 bytes at a time along the inner size: zero columns fill it up, and the
+                # normed rows are widened with zeros before the product
+                self._head_k = -(-self.hidden_size // 8) * 8
+                head = head.new_zeros(self.vocab_size, self._head_k)
+                head[:, :self.hidden_size] = self.head
+            self.head = ops.tile_weight(head)
 
     # --------------------------------------------------------------------- forward
     def forward(self, ctx, cache_views: dict[int, object]) -> Optional[torch.Tensor]:
@@ -234,5 +245,7 @@ class DecoderModel:
             h32 = torch.empty(h.shape, dtype=torch.float32, device=rt.device)
             ops.cast(h, h32)
             h = h32
+        if self._head_k != self.hidden_size:
+            h = ops.pad_cols(h, self._head_k)
         ops.gemm(h, self.head, logits)
         return logits

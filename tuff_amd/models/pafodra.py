@@ -69,4 +69,4 @@ def build_pafodra(cfg: PafodraConfig) -> DecoderModel:
     return DecoderModel(
         vocab_size=cfg.vocab, hidden_size=d, embedding=WeightDecl("embed", (cfg.vocab, d), "normal"),
         blocks=blocks, final_norm=_norm(d, "final.norm"), head=WeightDecl("head", (cfg.vocab, d), "normal"),
-        schedule=runs, max_positions=cfg.max_positions, embedding_scale=float(cfg.embedding["scale"]))
+        schedule=runs, max_positions=cfg.max_positions, embedding_scale=float(cfg.embedding["scale"]), pad_hidden=True)

@@ -200,10 +200,10 @@ class AttentionMixer(Mixer):
 
     def attend(self, q, o, ctx, cache, g) -> None:
         G = self.H // self.Hkv
-        if self.vd == self.hd and self.sinks is None and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
+        if self.vd == self.hd and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
             common = dict(block_table=g.block_table, req_info=ctx.req_info, H=self.H, Hkv=self.Hkv, hd=self.hd,
                           page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
-                          scale=self.scale)
+                          scale=self.scale, sinks=self.sinks)
             if ctx.max_q_len > 1:
                 # prompt portions in the step: blocks of columns walk over their keys through LDS.
                 # Requests with a single token beside them (runs of neighbours in the step's order) go

@@ -122,8 +122,8 @@ class GatedMLP(FeedForward):
         self.down.bind(weights, rt)
 
     def forward(self, h, ctx, residual, next_norm=None) -> None:
-        gu = self.gate_up.forward(h)
-        act = self.rt.empty(h.shape[0], self.width, dtype=gu.dtype)
+        gu = self.gate_up.forward(h, out_dtype=torch.float32)       # the activation reads the sums (and biases) as they are
+        act = self.rt.empty(h.shape[0], self.width)
         ops.glu(gu, act, self.activation)
         self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
 

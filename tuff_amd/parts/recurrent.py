@@ -68,9 +68,13 @@ class _LowRank:
         self.second.bind(padded, rt)
 
     def forward(self, x, out_dtype=None):
-        mid = self.first.forward(x)
-        if self.activation is not None:
-            ops.act_rows(mid, mid, self.activation)
+        if self.activation is None:
+            mid = self.first.forward(x)
+        else:
+            # the activation reads the product's float32 sums; what the second product takes is rounded once
+            raw = self.first.forward(x, out_dtype=torch.float32)
+            mid = torch.empty(raw.shape, dtype=self.first.rt.dtype, device=raw.device)
+            ops.act_rows(raw, mid, self.activation)
         return self.second.forward(mid, out_dtype=out_dtype)
 
 
@@ -132,7 +136,8 @@ class WkvMixer(Mixer):
         mixes = self.rt.empty(len(self.MIXES), T, self.d)
         ops.shift_mix(h, prev.state, self.mu, mixes, req_of_token=ctx.req_of_token, **step)
         ops.shift_state(h, prev.state, q_len=ctx.q_len, **step)
-        r, k, v, g = (self.proj[s].forward(mixes[i]) for i, s in enumerate(("r", "k", "v", "g")))
+        r, k, v = (self.proj[s].forward(mixes[i]) for i, s in enumerate(("r", "k", "v")))
+        g = self.proj["g"].forward(mixes[3], out_dtype=torch.float32)          # the gate's activation reads the sums as they are
         lw = self.decay.forward(mixes[4], out_dtype=torch.float32)
         o = torch.empty(T, HD, dtype=torch.float32, device=h.device)
         ops.wkv_scan(r, k, v, lw, self.w0, self.u, S.state, o, q_len=ctx.q_len, H=self.H, D=self.D, **step)
@@ -210,7 +215,7 @@ class GatedDeltaMixer(Mixer):
         q, k, v = (t.contiguous() for t in qkv.split([self.Cq, self.Cq, self.Cv], dim=1))
         b = self.beta.forward(h, out_dtype=torch.float32)
         a = self.decay.forward(h, out_dtype=torch.float32)
-        gate = self.gate.forward(h)
+        gate = self.gate.forward(h, out_dtype=torch.float32)
         o = torch.empty(T, self.Cv, dtype=torch.float32, device=h.device)
         ops.delta_scan(q, k, v, a, self.dt_bias, self.A_log, b, S.state, o, q_len=ctx.q_len, H=self.H, Hk=self.Hk,
                        D=self.D, Dv=self.Dv, **step)
