@@ -954,16 +954,20 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
         ws_ml = torch.empty(T * H * n_segs * 2, dtype=torch.float32, device=q.device)
     else:
         n_segs, seg_keys = 1, 0
-    _check(load("attention_prefill").tuff_attention_prefill_sinks(
-        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
-        block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk,
-        req_info.data_ptr(), H, Hkv, hd, page_size, int(window or 0), float(scale), n_segs, seg_keys,
-        None if ws_o is None else ws_o.data_ptr(), None if ws_ml is None else ws_ml.data_ptr(),
-        None if sinks is None else sinks.data_ptr(), _stream()), "attention_prefill")
-    if n_segs > 1:
-        _check(load("attention_mfma").tuff_attention_merge_sinks(
-            ws_o.data_ptr(), ws_ml.data_ptr(), out.data_ptr(), positions.data_ptr(), T, H, hd, int(window or 0), n_segs, seg_keys,
-            None if sinks is None else sinks.data_ptr(), _stream()), "attention_merge")
+    args = (q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+            block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk,
+            req_info.data_ptr(), H, Hkv, hd, page_size, int(window or 0), float(scale), n_segs, seg_keys,
+            None if ws_o is None else ws_o.data_ptr(), None if ws_ml is None else ws_ml.data_ptr())
+    merge = (ws_o.data_ptr(), ws_ml.data_ptr(), out.data_ptr(), positions.data_ptr(), T, H, hd, int(window or 0), n_segs,
+             seg_keys) if n_segs > 1 else None
+    if sinks is None:
+        _check(load("attention_prefill").tuff_attention_prefill(*args, _stream()), "attention_prefill")
+        if merge is not None:
+            _check(load("attention_mfma").tuff_attention_merge(*merge, _stream()), "attention_merge")
+    else:
+        _check(load("attention_prefill").tuff_attention_prefill_sinks(*args, sinks.data_ptr(), _stream()), "attention_prefill")
+        if merge is not None:
+            _check(load("attention_mfma").tuff_attention_merge_sinks(*merge, sinks.data_ptr(), _stream()), "attention_merge")
 
 
 def query_blocks(q_len, G: int, nb: int, ctx_len=None):
