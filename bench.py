@@ -335,6 +335,124 @@ def describe_shape(cfg, model) -> str:
             f"conv_L_cache {cfg.conv_L_cache}, {model.num_parameters()} parameters")
 
 
+# ------------------------------------------------------------- another design beside the closest model
+# Sizes that resemble a real model's layers, for `--design pafodra`: (width, layers, heads of 64 channels,
+# kv heads, dense feed-forward, experts, chosen, expert width).  The layer order repeats
+# [delta + dense, attention + experts, wkv + dense, wkv + experts].
+DESIGN_SIZES = {"1k": (1024, 8, 16, 4, 2816, 16, 2, 512), "2k": (2048, 8, 32, 8, 5632, 16, 2, 1024)}
+DESIGN_VOCAB = 32768
+
+
+def pafodra_config(size: str):
+    from tuff_amd.models.registry import config_from_dict
+    d, L, H, G, ff, E, top, eff = DESIGN_SIZES[size]
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "router": {"experts": E, "top": top}, "expert": {"ff": eff}, "shared": {"ff": eff}}
+    kinds = [
+        {"type": "channel_delta", "mixer": {"heads": H // 2, "kv_heads": H // 4, "dim": 64, "vdim": 128, "conv": 4}, "mlp": dense},
+        {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": 64, "vdim": 64, "scale": 0.125}, "mlp": moe},
+        {"type": "wkv", "mixer": {"heads": H, "dim": 64}, "mlp": dense},
+        {"type": "wkv", "mixer": {"heads": H, "dim": 64}, "mlp": moe},
+    ]
+    return config_from_dict({"architecture": "Pafodra", "vocab": DESIGN_VOCAB, "width": d, "embedding": {"scale": 1.0},
+                             "norm": {"eps": 1e-5}, "layers": [kinds[i % 4] for i in range(L)]})
+
+
+def lfm2_config_like(size: str):
+    """The LFM2 model of the same width, depth, heads, vocabulary and dense feed-forward: its short-conv
+    layers stand where the other design has its recurrences."""
+    from tuff_amd.models.registry import config_from_dict
+    d, L, H, G, ff, _, _, _ = DESIGN_SIZES[size]
+    return config_from_dict(dict(
+        architectures=["Lfm2ForCausalLM"], num_hidden_layers=L, full_attn_idxs=[i for i in range(L) if i % 4 == 1],
+        hidden_size=d, num_attention_heads=H, num_key_value_heads=G, block_ff_dim=ff, block_auto_adjust_ff_dim=False,
+        vocab_size=DESIGN_VOCAB, rope_theta=1000000.0, conv_L_cache=3, norm_eps=1e-5, tie_word_embeddings=False,
+        max_position_embeddings=32768))
+
+
+def time_design(cfg, dtype: str, prefill_tokens: int, batch: int, context: int, steps: int, classes: bool) -> dict:
+    """Prompts of `prefill_tokens` in one step each, and `steps` decode steps of `batch` requests at `context`
+    tokens, through Engine.step (recorded steps as served); tokens a second of both.  classes: the GPU time by
+    kernel class of one prompt step and one decode step (TUFF_TRACE must be set: nothing is recorded then)."""
+    import torch
+    from tuff_amd.csrc import ops
+    from tuff_amd.engine.batch import StepEntry
+    from tuff_amd.engine.engine import Engine
+    page = 16
+    pages = batch * (-(-(context + steps + 8) // page)) + 2 * (prefill_tokens // page) + 16
+    eng = Engine.from_config(cfg, SEED, dtype=dtype, page_size=page, num_pages=pages, max_requests=batch + 2)
+    g = torch.Generator().manual_seed(SEED)
+    V = eng.model.vocab_size
+    toks = lambda n: torch.randint(0, V, (n,), generator=g).tolist()
+    out = {"parameters": eng.model.num_parameters()}
+
+    def one_prompt():
+        eng.begin("p")
+        eng.step([StepEntry("p", toks(prefill_tokens), [prefill_tokens - 1])])
+        eng.end("p")
+    for _ in range(5):                                   # a step size that keeps coming is recorded at its third time
+        one_prompt()
+    torch.cuda.synchronize()
+    if classes:
+        ops.trace_reset()
+        one_prompt()
+        out["prefill_classes_us"] = {k: round(1e3 * v[1], 1) for k, v in sorted(ops.trace_stats().items(), key=lambda kv: -kv[1][1])}
+    t0 = time.perf_counter()
+    reps = 6
+    for _ in range(reps):
+        one_prompt()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    out.update(prefill_ms=round(1e3 * dt, 3), prefill_tok_s=round(prefill_tokens / dt, 1))
+
+    rids = [("d", b) for b in range(batch)]
+    for rid in rids:
+        eng.begin(rid)
+        left = context
+        while left > 0:
+            n = min(left, 2048)
+            eng.step([StepEntry(rid, toks(n), [])])
+            left -= n
+    step = lambda: eng.step([StepEntry(rid, toks(1), [0]) for rid in rids])
+    for _ in range(4):
+        step()
+    torch.cuda.synchronize()
+    if classes:
+        ops.trace_reset()
+        step()
+        out["decode_classes_us"] = {k: round(1e3 * v[1], 1) for k, v in sorted(ops.trace_stats().items(), key=lambda kv: -kv[1][1])}
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    elem = 2 if dtype == "bf16" else 4
+    read = eng.model.num_parameters() * elem + batch * (context * eng.layout.bytes_per_token(elem) + eng.layout.state_bytes_per_request())
+    out.update(decode_ms=round(1e3 * dt, 4), decode_tok_s=round(batch / dt, 1), decode_GBs=round(read / dt / 1e9, 1),
+               decode_roofline_frac=round(read / dt / 1e9 / HBM_PEAK_GBS, 4))
+    for rid in rids:
+        eng.end(rid)
+    return out
+
+
+def run_design(args) -> dict:
+    """`--design pafodra`: the Pafodra decoder at sizes that resemble a real model's layers (random weights)
+    beside the LFM2 decoder of equal width, depth and feed-forward."""
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    classes = os.environ.get("TUFF_TRACE", "")[:1] == "1"
+    out = {"design": "pafodra", "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_batch": args.batch,
+           "decode_context": args.design_context, "data": f"synthetic: seeded random weights (seed {SEED}), uniform random token ids",
+           "sizes": {}}
+    for size in args.design_sizes.split(","):
+        rec = {}
+        for name, cfg in (("pafodra", pafodra_config(size)), ("lfm2", lfm2_config_like(size))):
+            rec[name] = time_design(cfg, dtype, PREFILL_TOKENS, args.batch, args.design_context, args.point_steps, classes)
+        rec["prefill_ratio"] = round(rec["pafodra"]["prefill_tok_s"] / rec["lfm2"]["prefill_tok_s"], 3)
+        rec["decode_ratio"] = round(rec["pafodra"]["decode_tok_s"] / rec["lfm2"]["decode_tok_s"], 3)
+        out["sizes"][size] = rec
+    return out
+
+
 class Measured:
     """One engine of one shape and the points measured on it."""
 
@@ -413,6 +531,11 @@ def main() -> int:
     ap.add_argument("--shape", default="1.2b", choices=["1.2b"] + sorted(OTHER_SHAPES),
                     help="measure another shape of the architecture in the benchmark's place (for profiling; "
                          "its points only, no other shapes after it)")
+    ap.add_argument("--design", choices=["pafodra"],
+                    help="instead of the benchmark: prefill and decode of another design at sizes that resemble a real "
+                         "model's layers, beside the LFM2 model of equal size (TUFF_TRACE=1 adds GPU time by kernel class)")
+    ap.add_argument("--design-sizes", default="1k,2k", help="with --design: which of " + ",".join(sorted(DESIGN_SIZES)))
+    ap.add_argument("--design-context", type=int, default=2048, help="with --design: tokens every decoding request holds")
     ap.add_argument("--scenario", choices=sorted(SCENARIOS),
                     help="instead of the benchmark: a serving run through the scheduler on another shape")
     args = ap.parse_args()
@@ -422,6 +545,10 @@ def main() -> int:
     if int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; start it without a multi-process launcher")
         return 2
+
+    if args.design:
+        print(json.dumps(run_design(args)))
+        return 0
 
     if args.scenario:
         print(json.dumps(run_scenario(args.scenario, "bfloat16" if args.dtype == "bf16" else "float32", args.runs)))

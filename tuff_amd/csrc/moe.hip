@@ -18,11 +18,8 @@ __device__ __forceinline__ float act_fn(float z, int act) {
     return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-__global__ void route_kernel(const float* __restrict__ z, int stride, int* __restrict__ ids, float* __restrict__ wts,
-                             int n_tokens, int E, int top, int weight_fn) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n_tokens) return;
-    const float* row = z + (long long)t * stride;
+// The `top` largest of row[0..E-1] in the order (value descending, index ascending) and their weights.
+__device__ void choose(const float* row, int* ids, float* wts, long long t, int E, int top, int weight_fn) {
     float last = INFINITY;
     int last_id = -1;
     float zmax = 0.f, den = 0.f;
@@ -45,6 +42,39 @@ __global__ void route_kernel(const float* __restrict__ z, int stride, int* __res
     }
     if (weight_fn == 1)
         for (int s = 0; s < top; ++s) wts[(long long)t * top + s] /= den;
+}
+
+__global__ void route_kernel(const float* __restrict__ z, int stride, int* __restrict__ ids, float* __restrict__ wts,
+                             int n_tokens, int E, int top, int weight_fn) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_tokens) return;
+    choose(z + (long long)t * stride, ids, wts, t, E, top, weight_fn);
+}
+
+// Router logits and the choice in one kernel, a workgroup a token: z[t][n] = W[n] . h[t] in float32 (the
+// lanes of a wave take every 64th term and add their sums in a fixed butterfly, so a token's logits do not
+// depend on the step it is in), n < N rows of which the first E are experts (the rest: gates of other kinds
+// that are wanted as float32 products of the same rows).
+template <typename T>
+__global__ __launch_bounds__(256) void router_kernel(const T* __restrict__ h, const float* __restrict__ W, float* __restrict__ z,
+                                                     int* __restrict__ ids, float* __restrict__ wts, int d, int N, int E,
+                                                     int top, int weight_fn) {
+    extern __shared__ float sm[];
+    float* xs = sm;
+    float* zs = sm + d;
+    const long long t = blockIdx.x;
+    for (int c = threadIdx.x; c < d; c += 256) xs[c] = to_f32(h[t * d + c]);
+    __syncthreads();
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    for (int n = wave; n < N; n += 4) {
+        const float* wr = W + (long long)n * d;
+        float acc = 0.f;
+        for (int c = lane; c < d; c += WAVE) acc = fmaf(wr[c], xs[c], acc);
+        acc = wave_sum(acc);
+        if (lane == 0) { zs[n] = acc; z[t * N + n] = acc; }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) choose(zs, ids, wts, t, E, top, weight_fn);
 }
 
 constexpr int ROWS_WG = 16;          // output rows a workgroup of four waves computes
@@ -104,6 +134,117 @@ __global__ void combine_kernel(const float* __restrict__ y, const float* __restr
     }
     residual[i] += acc;
 }
+
+// ------------------------------------------------------------ many rows: grouped by expert, matrix cores
+typedef __bf16 bf16x8_ __attribute__((ext_vector_type(8)));
+constexpr int GROUP_MAX_E = 1024;
+
+// One workgroup sorts the rows (token, choice) by expert and cuts each expert's rows into tiles of TM:
+// sorted[pos] = row; tiles[i] = (expert, first pos, rows), expert -1 for tiles beyond the last.  The order of an
+// expert's rows among themselves is whatever the atomics give: no row's result depends on its place in a tile.
+__global__ __launch_bounds__(1024) void group_rows_kernel(const int* __restrict__ ids, int R, int E, int TM, int* __restrict__ sorted,
+                                                          int* __restrict__ tiles, int max_tiles) {
+    __shared__ int cnt[GROUP_MAX_E], off[GROUP_MAX_E], cur[GROUP_MAX_E];
+    for (int e = threadIdx.x; e < E; e += 1024) { cnt[e] = 0; cur[e] = 0; }
+    __syncthreads();
+    for (int r = threadIdx.x; r < R; r += 1024) atomicAdd(&cnt[ids[r]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int o = 0, nt = 0;
+        for (int e = 0; e < E; ++e) {
+            off[e] = o;
+            for (int p = 0; p < cnt[e] && nt < max_tiles; p += TM, ++nt) {
+                tiles[3 * nt] = e; tiles[3 * nt + 1] = o + p; tiles[3 * nt + 2] = min(TM, cnt[e] - p);
+            }
+            o += cnt[e];
+        }
+        for (; nt < max_tiles; ++nt) { tiles[3 * nt] = -1; tiles[3 * nt + 1] = 0; tiles[3 * nt + 2] = 0; }
+    }
+    __syncthreads();
+    for (int r = threadIdx.x; r < R; r += 1024) {
+        const int e = ids[r];
+        sorted[off[e] + atomicAdd(&cur[e], 1)] = r;
+    }
+}
+
+__device__ __forceinline__ f32x4 mfma16(bf16x8_ a, bf16x8_ b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// A tile of up to 16 TMT rows of one expert times a slice of that expert's matrix.  W: every expert's matrix
+// [N][K] in blocks of 16 rows x 32 k in the order of the matrix cores' first operand ([E][ceil(N/16)][ceil(K/32)]
+// blocks of 1 KB: piece l = row l % 16, k 8 (l / 16) .. + 7); a wave takes NF blocks of rows, the four waves of a
+// workgroup neighbouring ones.  UP: the rows are tokens of h gathered through `sorted` (row / top), times the
+// choice's weight and rounded where scale_input; the result act(.) goes to A [R][N] in sorted order.  Else: the
+// rows are A's, in place, and the float32 result goes to Y [R][N] at the row's own number.
+template <int NF, int TMT, bool UP>
+__global__ __launch_bounds__(256) void grouped_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                      const int* __restrict__ tiles, const int* __restrict__ sorted,
+                                                      const float* __restrict__ wts, bf16_t* __restrict__ A, float* __restrict__ Y,
+                                                      int K, int N, int top, int act, int scale_input) {
+    const int tile = blockIdx.x;
+    const int e = tiles[3 * tile];
+    if (e < 0) return;
+    const int pos0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, n16 = lane % 16, g = lane / 16;
+    const int NT16 = (N + 15) / 16, KB = (K + 31) / 32;
+    const int ft0 = (blockIdx.y * 4 + wave) * NF;
+    if (ft0 >= NT16) return;
+    long long src[TMT];
+    int own[TMT];
+    float scale[TMT];
+    bool valid[TMT];
+#pragma unroll
+    for (int tt = 0; tt < TMT; ++tt) {
+        const int idx = tt * 16 + n16;
+        valid[tt] = idx < rows;
+        own[tt] = valid[tt] ? sorted[pos0 + idx] : 0;
+        src[tt] = UP ? own[tt] / top : pos0 + idx;
+        scale[tt] = (UP && scale_input && valid[tt]) ? wts[own[tt]] : 1.f;
+    }
+    f32x4 acc[NF][TMT];
+#pragma unroll
+    for (int nf = 0; nf < NF; ++nf)
+#pragma unroll
+        for (int tt = 0; tt < TMT; ++tt) acc[nf][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const bf16x8_ zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bf16_t* We = W + (long long)e * NT16 * KB * 512;
+    constexpr int UN = NF == 1 ? 8 : 2;        // few registers a step: more loads under way (narrow tiles stream the weights)
+#pragma unroll UN
+    for (int kb = 0; kb < KB; ++kb) {
+        const int k = kb * 32 + 8 * g;
+        bf16x8_ xb[TMT];
+#pragma unroll
+        for (int tt = 0; tt < TMT; ++tt) {
+            xb[tt] = (valid[tt] && k < K) ? *(const bf16x8_*)(X + src[tt] * K + k) : zero;
+            if (UP && scale_input) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xb[tt][i] = (bf16_t)((float)xb[tt][i] * scale[tt]);
+            }
+        }
+#pragma unroll
+        for (int nf = 0; nf < NF; ++nf) {
+            if (ft0 + nf < NT16) {
+                const bf16x8_ wa = *(const bf16x8_*)(We + (((long long)(ft0 + nf) * KB + kb) * 64 + lane) * 8);
+#pragma unroll
+                for (int tt = 0; tt < TMT; ++tt) acc[nf][tt] = mfma16(wa, xb[tt], acc[nf][tt]);
+            }
+        }
+    }
+#pragma unroll
+    for (int nf = 0; nf < NF; ++nf)
+#pragma unroll
+        for (int tt = 0; tt < TMT; ++tt) {
+            if (!valid[tt] || ft0 + nf >= NT16) continue;
+            const int col = (ft0 + nf) * 16 + 4 * g;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (col + i >= N) continue;
+                if (UP) A[(long long)(pos0 + tt * 16 + n16) * N + col + i] = (bf16_t)act_fn(acc[nf][tt][i], act);
+                else Y[(long long)own[tt] * N + col + i] = acc[nf][tt][i];
+            }
+        }
+}
 }  // namespace
 
 TUFF_EXPORT int tuff_moe_route(const float* z, int stride, int* ids, float* wts, int n_tokens, int E, int top, int weight_fn,
@@ -136,5 +277,51 @@ TUFF_EXPORT int tuff_moe_experts(const void* h, const void* w_up, const void* w_
     }
     const long long n = (long long)n_tokens * d;
     hipLaunchKernelGGL(combine_kernel, dim3((unsigned)ceil_div_ll(n, 256)), block, 0, stream, y, wts, residual, n, d, top, !scale_input);
+    return launch_status();
+}
+
+// z float32 [T][N], the first E columns the experts' logits; ids, wts [T][top].  W float32 [N][d]; h [T][d] of type dt.
+TUFF_EXPORT int tuff_moe_router(const void* h, int dt, const float* W, float* z, int* ids, float* wts, int n_tokens, int d,
+                                int N, int E, int top, int weight_fn, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (top < 1 || top > E || N < E || (long long)(d + N) * 4 > 65536) return -2;
+    const size_t lds = (size_t)(d + N) * sizeof(float);
+    if (dt == DT_F32) hipLaunchKernelGGL(router_kernel<float>, dim3(n_tokens), dim3(256), lds, stream, (const float*)h, W, z, ids, wts, d, N, E, top, weight_fn);
+    else hipLaunchKernelGGL(router_kernel<bf16_t>, dim3(n_tokens), dim3(256), lds, stream, (const bf16_t*)h, W, z, ids, wts, d, N, E, top, weight_fn);
+    return launch_status();
+}
+
+// Rows a tile of tuff_moe_experts_grouped holds for R rows over E experts, and the tiles it may need.
+TUFF_EXPORT int tuff_moe_grouped_tile_rows(long long R, int E) { return R >= 24ll * E ? 32 : 16; }
+
+// The experts of many rows on the matrix cores (bfloat16): h [T][d]; w_up, w_down every expert's matrix in blocks
+// (see grouped_kernel), [E][F x d] and [E][d x F]; ids, wts [T][top]; work arrays sorted int32 [T*top], tiles int32
+// [3 * max_tiles] with max_tiles >= ceil(T*top / tile rows) + E, a bfloat16 [T*top][F], y float32 [T*top][d];
+// residual float32 [T][d].  d and F multiples of 8, E at most 1024.
+TUFF_EXPORT int tuff_moe_experts_grouped(const void* h, const void* w_up, const void* w_down, const int* ids, const float* wts,
+                                         int* sorted, int* tiles, int max_tiles, void* a, float* y, float* residual,
+                                         int n_tokens, int d, int F, int E, int top, int act, int scale_input, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    const long long R = (long long)n_tokens * top;
+    if (d % 8 || F % 8 || E > GROUP_MAX_E || E < 1 || R > 0x7fffffffll) return -2;
+    const int TM = tuff_moe_grouped_tile_rows(R, E);
+    if (max_tiles < (int)((R + TM - 1) / TM) + E) return -2;
+    hipLaunchKernelGGL(group_rows_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)R, E, TM, sorted, tiles, max_tiles);
+    const bf16_t* H_ = (const bf16_t*)h;
+    bf16_t* A_ = (bf16_t*)a;
+    // few rows an expert: many narrow workgroups stream the weights; many: wide ones reuse them
+    if (TM == 32) {
+        hipLaunchKernelGGL((grouped_kernel<4, 2, true>), dim3(max_tiles, ceil_div(ceil_div(F, 16), 16)), dim3(256), 0, stream,
+                           H_, (const bf16_t*)w_up, tiles, sorted, wts, A_, nullptr, d, F, top, act, scale_input);
+        hipLaunchKernelGGL((grouped_kernel<4, 2, false>), dim3(max_tiles, ceil_div(ceil_div(d, 16), 16)), dim3(256), 0, stream,
+                           A_, (const bf16_t*)w_down, tiles, sorted, wts, nullptr, y, F, d, top, act, scale_input);
+    } else {
+        hipLaunchKernelGGL((grouped_kernel<1, 1, true>), dim3(max_tiles, ceil_div(ceil_div(F, 16), 4)), dim3(256), 0, stream,
+                           H_, (const bf16_t*)w_up, tiles, sorted, wts, A_, nullptr, d, F, top, act, scale_input);
+        hipLaunchKernelGGL((grouped_kernel<1, 1, false>), dim3(max_tiles, ceil_div(ceil_div(d, 16), 4)), dim3(256), 0, stream,
+                           A_, (const bf16_t*)w_down, tiles, sorted, wts, nullptr, y, F, d, top, act, scale_input);
+    }
+    const long long n = (long long)n_tokens * d;
+    hipLaunchKernelGGL(combine_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, y, wts, residual, n, d, top, !scale_input);
     return launch_status();
 }

@@ -55,6 +55,11 @@ _SIGNATURES = {
     },
     "moe": {
         "tuff_moe_route": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_moe_router": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                            _c_int, _c_void_p],
+        "tuff_moe_grouped_tile_rows": [_c_ll, _c_int],
+        "tuff_moe_experts_grouped": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                                     _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_moe_experts": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
@@ -1153,6 +1158,59 @@ def moe_route(z, ids, wts, *, E, top, weights: str = "sigmoid") -> None:
     _check(load("moe").tuff_moe_route(z.data_ptr(), z.shape[1], _gpu("ids", ids, torch.int32, (T, top)),
                                       _gpu("wts", wts, torch.float32, (T, top)), T, E, top,
                                       {"sigmoid": 0, "softmax": 1}[weights], _stream()), "moe_route")
+
+
+ROUTER_MAX_FLOATS = 16384          # hidden size + logits a token: what the router kernel keeps in LDS
+
+
+def moe_router(h, w, z, ids, wts, *, E, top, weights: str = "sigmoid") -> None:
+    """z = h @ w.T in float32 (h [T, d] of the compute type, w float32 [N, d], z float32 [T, N]) and, of its first
+    E columns, the choice as moe_route makes it, in one kernel."""
+    T, d = h.shape
+    N = w.shape[0]
+    if d + N > ROUTER_MAX_FLOATS:
+        raise KernelError(f"moe_router: hidden size {d} + {N} logits above {ROUTER_MAX_FLOATS}")
+    _check(load("moe").tuff_moe_router(_gpu("h", h), _dt(h), _gpu("w", w, torch.float32, (N, d)), _gpu("z", z, torch.float32, (T, N)),
+                                       _gpu("ids", ids, torch.int32, (T, top)), _gpu("wts", wts, torch.float32, (T, top)),
+                                       T, d, N, E, top, {"sigmoid": 0, "softmax": 1}[weights], _stream()), "moe_router")
+
+
+def tile_experts(ws) -> torch.Tensor:
+    """Every expert's bfloat16 matrix [N, K] in the order tile_weight gives one, stacked: [E, ceil(N/16), ceil(K/32), 64, 8]."""
+    return torch.stack([tile_weight(w).blocks for w in ws]).contiguous()
+
+
+def moe_grouped_supported(dtype, d: int, F: int, E: int) -> bool:
+    return dtype == torch.bfloat16 and d % 8 == 0 and F % 8 == 0 and 1 <= E <= 1024
+
+
+def moe_experts_grouped(h, up_tiles, down_tiles, ids, wts, residual, *, F: int, activation: str = "relu2",
+                        scale_input: bool = True) -> None:
+    """moe_experts on the matrix cores, bfloat16: the rows (token, choice) are sorted by expert and every expert's
+    rows go through its two matrices in tiles.  up_tiles, down_tiles: tile_experts() of the [F, d] and [d, F] matrices."""
+    T, d = h.shape
+    E, top = up_tiles.shape[0], ids.shape[1]
+    if not moe_grouped_supported(h.dtype, d, F, E):
+        raise KernelError(f"moe_experts_grouped: bfloat16, sizes that are multiples of 8 and at most 1024 experts; got {h.dtype}, {d}, {F}, {E}")
+    _gpu("h", h, torch.bfloat16)
+    _gpu("up_tiles", up_tiles, torch.bfloat16, (E, -(-F // 16), -(-d // 32), 64, 8))
+    _gpu("down_tiles", down_tiles, torch.bfloat16, (E, -(-d // 16), -(-F // 32), 64, 8))
+    _gpu("ids", ids, torch.int32, (T, top))
+    _gpu("wts", wts, torch.float32, (T, top))
+    _gpu("residual", residual, torch.float32, (T, d))
+    R = T * top
+    lib = load("moe")
+    max_tiles = -(-R // int(lib.tuff_moe_grouped_tile_rows(R, E))) + E
+    dev = h.device
+    srt = torch.empty(R, dtype=torch.int32, device=dev)
+    tiles = torch.empty(3 * max_tiles, dtype=torch.int32, device=dev)
+    a = torch.empty(R, F, dtype=torch.bfloat16, device=dev)
+    y = torch.empty(R, d, dtype=torch.float32, device=dev)
+    _check(lib.tuff_moe_experts_grouped(h.data_ptr(), up_tiles.data_ptr(), down_tiles.data_ptr(), ids.data_ptr(), wts.data_ptr(),
+                                        srt.data_ptr(), tiles.data_ptr(), max_tiles, a.data_ptr(), y.data_ptr(),
+                                        residual.data_ptr(), T, d, F, E, top,
+                                        {"relu2": 0, "silu": 1, "gelu_tanh": 2}[activation], int(scale_input), _stream()),
+           "moe_experts_grouped")
 
 
 def moe_experts(h, w_up, w_down, ids, wts, residual, *, activation: str = "relu2", scale_input: bool = True) -> None:

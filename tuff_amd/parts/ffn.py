@@ -156,8 +156,6 @@ class MoE(FeedForward):
             raise ValueError("one (up, down) pair of names per expert")
         self.Fs = int(shared_dim)
         self.shared_gate = self.Fs > 0 and "shared.sg" in self.names
-        rows = [self.names["router"]] + ([self.names["shared.sg"]] if self.shared_gate else [])
-        self.router = Linear(rows, self.d, [self.E] + ([1] if self.shared_gate else []), float32=True)
         self.shared_up = self.shared_down = None
         if self.Fs:
             self._make_shared(self.Fs)
@@ -167,7 +165,9 @@ class MoE(FeedForward):
         self.shared_down = Linear(self.names["shared.down"], width, self.d)
 
     def weight_decls(self):
-        decls = self.router.weight_decls()
+        decls = [WeightDecl(self.names["router"], (self.E, self.d), "normal", role="projection")]
+        if self.shared_gate:
+            decls.append(WeightDecl(self.names["shared.sg"], (1, self.d), "normal", role="projection"))
         for up, down in self.names["experts"]:
             decls += [WeightDecl(up, (self.F, self.d), "normal", role="projection"),
                       WeightDecl(down, (self.d, self.F), "normal", role="projection")]
@@ -177,13 +177,22 @@ class MoE(FeedForward):
         return decls
 
     def kernel_modules(self):
-        return ["moe", "elementwise", "gemm_f32"]
+        return ["moe", "elementwise"]
 
     def bind(self, weights, rt: Runtime):
         self.rt = rt
-        self.router.bind(weights, rt)
-        self.w_up = torch.stack([weights[up] for up, _ in self.names["experts"]]).contiguous()           # [E, F, d]
-        self.w_down = torch.stack([weights[down] for _, down in self.names["experts"]]).contiguous()     # [E, d, F]
+        # the router's rows (and the shared expert's gate row behind them) stay float32: their products decide
+        rows = [weights[self.names["router"]]] + ([weights[self.names["shared.sg"]]] if self.shared_gate else [])
+        self.router_w = torch.cat([r.to(torch.float32).reshape(-1, self.d) for r in rows]).contiguous()
+        ups = [weights[up] for up, _ in self.names["experts"]]
+        downs = [weights[down] for _, down in self.names["experts"]]
+        self.grouped = ops.moe_grouped_supported(ups[0].dtype, self.d, self.F, self.E) and rt.dtype == torch.bfloat16
+        if self.grouped:
+            # the matrix cores' order, an expert after the other
+            self.up_tiles, self.down_tiles = ops.tile_experts(ups), ops.tile_experts(downs)
+        else:
+            self.w_up = torch.stack(ups).contiguous()                # [E, F, d]
+            self.w_down = torch.stack(downs).contiguous()            # [E, d, F]
         if self.Fs:
             up, down = weights[self.names["shared.up"]], weights[self.names["shared.down"]]
             if self.Fs % 8 and up.dtype == torch.bfloat16 and down.dtype == torch.bfloat16:
@@ -197,12 +206,16 @@ class MoE(FeedForward):
 
     def forward(self, h, ctx, residual) -> None:
         T = h.shape[0]
-        z = self.router.forward(h, out_dtype=torch.float32)                  # [T, E (+ 1)]
+        z = torch.empty(T, self.router_w.shape[0], dtype=torch.float32, device=h.device)        # [T, E (+ 1)]
         ids = torch.empty(T, self.top, dtype=torch.int32, device=h.device)
         wts = torch.empty(T, self.top, dtype=torch.float32, device=h.device)
-        ops.moe_route(z, ids, wts, E=self.E, top=self.top, weights=self.router_weights)
-        ops.moe_experts(h, self.w_up, self.w_down, ids, wts, residual, activation=self.activation,
-                        scale_input=self.scale_input)
+        ops.moe_router(h, self.router_w, z, ids, wts, E=self.E, top=self.top, weights=self.router_weights)
+        if self.grouped:
+            ops.moe_experts_grouped(h, self.up_tiles, self.down_tiles, ids, wts, residual, F=self.F,
+                                    activation=self.activation, scale_input=self.scale_input)
+        else:
+            ops.moe_experts(h, self.w_up, self.w_down, ids, wts, residual, activation=self.activation,
+                            scale_input=self.scale_input)
         if self.Fs:
             a = self.shared_up.forward(h)
             # the gate is one number a token and the second product is linear: it goes onto the activations
