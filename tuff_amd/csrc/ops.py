@@ -46,10 +46,11 @@ _SIGNATURES = {
         "tuff_shift_state": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tuff_conv_act": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
-        "tuff_wkv_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_wkv_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                          _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_delta_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                            _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                            _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                            _c_int, _c_int, _c_int, _c_void_p],
         "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int,
                                 _c_float, _c_void_p],
     },
@@ -1101,8 +1102,8 @@ SCAN_MAX_DIM = 256
 def wkv_scan(r, k, v, lw, w0, u, state, out, *, q_start, q_len, state_slot, H, D) -> None:
     """The decaying outer-product recurrence over each request's tokens of the step, from and to
     state[slot] (float32 [slots, H, D, D]): o = (S + diag(u) k v^T)^T r, then S = diag(w) S + k v^T with
-    w = exp(-exp(lw + w0)).  r, k, v [T, H * D]; lw float32 [T, H * D]; w0 float32 [H * D]; u float32 [H, D];
-    out float32 [T, H * D]."""
+    w = exp(-exp(lw + w0)).  r, k, v [T, H * D]; lw float32 [T, H * D] (overwritten with the decays); w0 float32
+    [H * D]; u float32 [H, D]; out float32 [T, H * D]."""
     T = r.shape[0]
     R = q_start.shape[0]
     dt = r.dtype
@@ -1111,28 +1112,32 @@ def wkv_scan(r, k, v, lw, w0, u, state, out, *, q_start, q_len, state_slot, H, D
     _check(load("recurrent").tuff_wkv_scan(
         _gpu("r", r, shape=(T, H * D)), _gpu("k", k, dt, (T, H * D)), _gpu("v", v, dt, (T, H * D)), _dt(r),
         _gpu("lw", lw, torch.float32, (T, H * D)), _gpu("w0", w0, torch.float32, (H * D,)), _gpu("u", u, torch.float32, (H, D)),
+        torch.empty(T, H, dtype=torch.float32, device=r.device).data_ptr(),
         _gpu("state", state, torch.float32, (None, H, D, D)), _gpu("out", out, torch.float32, (T, H * D)),
         _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
-        _gpu("state_slot", state_slot, torch.int32, (R,)), R, H, D, _stream()), "wkv_scan")
+        _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, D, _stream()), "wkv_scan")
 
 
 def delta_scan(q, k, v, a, dt_bias, A_log, b, state, out, *, q_start, q_len, state_slot, H, Hk, D, Dv) -> None:
     """The gated delta rule over each request's tokens of the step, from and to state[slot] (float32
     [slots, H, D, Dv]): S = g S; e = beta (v - S^T k); S = S + k e^T; o = S^T q, with q and k made unit
     vectors per head (q also times D^-1/2), g = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b).
-    q, k [T, Hk * D]; v [T, H * Dv]; a float32 [T, H * D]; b float32 [T, H]; out float32 [T, H * Dv]."""
+    q, k [T, Hk * D]; v [T, H * Dv]; a float32 [T, H * D] (overwritten with the decays); b float32 [T, H]; out
+    float32 [T, H * Dv]."""
     T = q.shape[0]
     R = q_start.shape[0]
     dt = q.dtype
     if D > SCAN_MAX_DIM or Hk < 1 or H % Hk:
         raise KernelError(f"delta_scan: key size {D} (at most {SCAN_MAX_DIM}) / heads {H}:{Hk} not supported")
+    work = torch.empty(2, T, H * D, dtype=torch.float32, device=q.device)       # q and k as unit vectors
     _check(load("recurrent").tuff_delta_scan(
         _gpu("q", q, shape=(T, Hk * D)), _gpu("k", k, dt, (T, Hk * D)), _gpu("v", v, dt, (T, H * Dv)), _dt(q),
         _gpu("a", a, torch.float32, (T, H * D)), _gpu("dt_bias", dt_bias, torch.float32, (H * D,)),
         _gpu("A_log", A_log, torch.float32, (H,)), _gpu("b", b, torch.float32, (T, H)),
+        work[0].data_ptr(), work[1].data_ptr(), torch.empty(T, H, dtype=torch.float32, device=q.device).data_ptr(),
         _gpu("state", state, torch.float32, (None, H, D, Dv)), _gpu("out", out, torch.float32, (T, H * Dv)),
         _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
-        _gpu("state_slot", state_slot, torch.int32, (R,)), R, H, Hk, D, Dv, _stream()), "delta_scan")
+        _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, Hk, D, Dv, _stream()), "delta_scan")
 
 
 def head_norm_gate(o, w, gate, out, *, H, Dv, eps, per_head_weight: bool, gate_activation: Optional[str]) -> None:

@@ -102,160 +102,233 @@ __global__ void conv_state_kernel(const T* __restrict__ x, float* __restrict__ s
 }
 
 // ------------------------------------------------------------------------ recurrences
-// One wave per (request, head, 64 value channels): lane j keeps column j of the head's state,
-// S[0..D-1][j], in registers (NI = ceil(D / 4) groups of four rows) and walks the request's tokens in
-// order.  What a token brings for the key channels (r or q, k, the decay) is staged by the wave
-// through LDS, the token after it is fetched while the current one is computed.
+// Two kernels.  The first works on all tokens at once, a wave a (token, head): what enters the recurrence
+// besides the projected rows is made there in float32, the decay w = exp(-exp(lw + w0)) and the bonus
+// sum_i r_i u_i k_i (wkv), or the decay g = exp(-exp(A_log) softplus(a + dt_bias)), the write strength
+// sigmoid(b) and q and k as unit vectors per head (x / sqrt(sum x^2 + 1e-6), q also times D^-1/2) (delta).
 //
-// wkv:    o_j = sum_i r_i (S_ij + u_i k_i v_j);   S_ij <- w_i S_ij + k_i v_j
-//         w_i = exp(-exp(lw_i + w0_i))
+// The second walks each request's tokens in order, one wave per (request, head, a few value channels).  SPLIT
+// neighbouring lanes (4 for key sizes up to 32, else 16) share a value channel j and keep a share of the state's
+// column S[0..D-1][j] each in registers (RP rows); their partial sums meet in exchanges inside the group, always
+// in the same order.  A token is a chain of dependent steps for a wave, so what a wave does for a token is kept
+// short and the head's columns are spread over many waves.
+// Eight tokens at a time: what they bring for the key channels is fetched while the eight before are computed
+// and staged through LDS, from where every lane reads it as broadcasts.  The arithmetic of a token is the same
+// whatever the step holds, so the result does not depend on how a sequence was cut.
+//
+// wkv:    o_j = sum_i r_i S_ij + bonus v_j;   S_ij <- w_i S_ij + k_i v_j
 // delta:  S_ij <- g_i S_ij;  e_j = beta (v_j - sum_i k_i S_ij);  S_ij <- S_ij + k_i e_j;  o_j = sum_i q_i S_ij
-//         g_i = exp(-exp(A_log) softplus(a_i + dt_bias_i)), beta = sigmoid(b), q and k unit vectors
-//         (x / sqrt(sum x^2 + 1e-6)), q also times D^(-1/2)
-struct ScanArgs {
-    const void *a, *k, *v;          // per token: r or q [T][Ha*D], k [T][Ha*D], v [T][H*Dv]   (Ha: heads of a and k)
-    const float* decay_in;          // per token [T][H*D]: lw (wkv) or a (delta)
+struct PrepArgs {
+    const void *a, *k;              // r or q, k [T][Ha*D] of the compute type
+    float* decay;                   // in: lw or a [T][H*D]; out, in place: w or g
     const float* decay_bias;        // [H*D]: w0 or dt_bias
     const float* per_head;          // wkv: u [H][D];  delta: A_log [H]
     const float* beta_in;           // delta: b [T][H]
+    float *qn, *kn;                 // delta, out: unit vectors [T][H][D]
+    float* scalar;                  // out [T][H]: bonus (wkv) or beta (delta)
+    int H, Ha, D;
+};
+
+template <typename T, bool DELTA>
+__global__ __launch_bounds__(WAVE) void scan_prep_kernel(PrepArgs p) {
+    const long long t = blockIdx.x;
+    const int head = blockIdx.y, lane = threadIdx.x;
+    const int D = p.D, H = p.H, Ha = p.Ha;
+    const int ha = head / (H / Ha);
+    const T* pa = (const T*)p.a + (t * Ha + ha) * D;
+    const T* pk = (const T*)p.k + (t * Ha + ha) * D;
+    float* dec = p.decay + (t * H + head) * D;
+    if (DELTA) {
+        float qq = 0.f, kk = 0.f;
+        for (int i = lane; i < D; i += WAVE) {
+            const float q = to_f32(pa[i]), k = to_f32(pk[i]);
+            qq = fmaf(q, q, qq);
+            kk = fmaf(k, k, kk);
+        }
+        qq = wave_sum(qq); kk = wave_sum(kk);
+        const float qn = (1.0f / sqrtf((float)D)) / sqrtf(qq + 1e-6f), kn = 1.0f / sqrtf(kk + 1e-6f);
+        const float neg_rate = -expf(p.per_head[head]);
+        for (int i = lane; i < D; i += WAVE) {
+            p.qn[(t * H + head) * D + i] = to_f32(pa[i]) * qn;
+            p.kn[(t * H + head) * D + i] = to_f32(pk[i]) * kn;
+            dec[i] = expf(neg_rate * softplusf_(dec[i] + p.decay_bias[head * D + i]));
+        }
+        if (lane == 0) p.scalar[t * H + head] = sigmoidf_(p.beta_in[t * H + head]);
+    } else {
+        float bonus = 0.f;
+        for (int i = lane; i < D; i += WAVE) {
+            bonus = fmaf(to_f32(pa[i]) * p.per_head[head * D + i], to_f32(pk[i]), bonus);
+            dec[i] = expf(-expf(dec[i] + p.decay_bias[head * D + i]));
+        }
+        bonus = wave_sum(bonus);
+        if (lane == 0) p.scalar[t * H + head] = bonus;
+    }
+}
+
+struct ScanArgs {
+    const void *a, *k, *v;          // per token: a (r, or unit q) and k [T][Ha*D], v [T][H*Dv]   (Ha: heads of a and k)
+    const float* decay;             // per token [T][H*D]: w or g
+    const float* scalar;            // per token [T][H]: bonus or beta
     float* state;                   // [slots][H][D][Dv]
     float* out;                     // [T][H][Dv]
     const int *q_start, *q_len, *state_slot;
     int H, Ha, D, Dv;
 };
 
-template <typename T, int NI, bool DELTA>
+constexpr int SCAN_CH = 8;          // tokens staged at a time
+
+// The sum over the SPLIT neighbouring lanes that share a value channel, the same in all of them: exchanges
+// inside a quad (lane ^ 1, then lane ^ 2) and, for 16, rotations by 4 and by 8 within the row of 16 lanes.
+template <int CTRL>
+__device__ __forceinline__ float dpp_of(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int SPLIT>
+__device__ __forceinline__ float group_sum(float v) {
+    v += dpp_of<0xB1>(v);
+    v += dpp_of<0x4E>(v);
+    if (SPLIT == 16) {
+        v += dpp_of<0x124>(v);
+        v += dpp_of<0x128>(v);
+    }
+    return v;
+}
+
+// TA: type of a and k (the compute type for wkv's r and k, float for the delta rule's unit vectors); T: type of v.
+template <typename TA, typename T, int NI16, int SPLIT, bool DELTA>
 __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
-    constexpr int DP = NI * 4;                         // key channels, padded
+    constexpr int RP = NI16 * 4;                       // rows of the state's column a lane keeps
+    constexpr int DP = RP * SPLIT;                     // key channels, padded
+    constexpr int SCAN_COLS = WAVE / SPLIT;            // value channels a wave
     constexpr int PER = (DP + WAVE - 1) / WAVE;        // key channels a lane stages
-    __shared__ __attribute__((aligned(16))) float sa[2][DP];
-    __shared__ __attribute__((aligned(16))) float sk[2][DP];
-    __shared__ __attribute__((aligned(16))) float sw[2][DP];
+    constexpr int CH = SCAN_CH;
+    __shared__ __attribute__((aligned(16))) float sa[CH][DP];
+    __shared__ __attribute__((aligned(16))) float sk[CH][DP];
+    __shared__ __attribute__((aligned(16))) float sw[CH][DP];
     const int r = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const int n = p.q_len[r];
     if (n <= 0) return;
     const int D = p.D, Dv = p.Dv, H = p.H, Ha = p.Ha;
     const int ha = head / (H / Ha);
-    const int j = blockIdx.z * WAVE + lane;
+    const int part = lane % SPLIT;
+    const int j = blockIdx.z * SCAN_COLS + lane / SPLIT;
     const bool jv = j < Dv;
+    const int row0 = part * RP;
     const int t0 = p.q_start[r];
     float* S = p.state + (((long long)p.state_slot[r] * H + head) * D) * Dv + j;
-    const T* pa = (const T*)p.a;
-    const T* pk = (const T*)p.k;
+    const TA* pa = (const TA*)p.a;
+    const TA* pk = (const TA*)p.k;
     const T* pv = (const T*)p.v;
 
-    float s[DP];
+    float s[RP];
 #pragma unroll
-    for (int i = 0; i < DP; ++i) s[i] = (jv && i < D) ? S[(long long)i * Dv] : 0.f;
+    for (int i = 0; i < RP; ++i) s[i] = (jv && row0 + i < D) ? S[(long long)(row0 + i) * Dv] : 0.f;
 
-    float bias[PER], extra[PER];
+    // what the next eight tokens bring
+    // (kept as they were loaded: a conversion on the spot would wait for the load)
+    TA fa[CH][PER], fk[CH][PER];
+    T fv[CH];
+    float fw[CH][PER], fb[CH];
+    // Every load is issued whatever the lane and token (from a clamped place where there is nothing to fetch);
+    // what does not count is replaced when the values are staged, eight tokens later: a load inside a condition
+    // would be waited for on the spot, and so would a value that is looked at right after its load.
+    const int jc = min(j, Dv - 1);
+    auto fetch = [&](int first, int count) {
 #pragma unroll
-    for (int e = 0; e < PER; ++e) {
-        const int i = lane + e * WAVE;
-        bias[e] = i < D ? p.decay_bias[head * D + i] : 0.f;
-        extra[e] = (!DELTA && i < D) ? p.per_head[head * D + i] : 0.f;      // u
-    }
-    const float neg_rate = DELTA ? -expf(p.per_head[head]) : 0.f;
-    const float q_scale = DELTA ? 1.0f / sqrtf((float)D) : 1.f;
-
-    // what a token brings, fetched one token ahead
-    float fa[PER], fk[PER], fw[PER], fv = 0.f, fb = 0.f;
-    auto fetch = [&](int t) {
+        for (int tt = 0; tt < CH; ++tt) {
+            const long long t = first + min(tt, count - 1);
 #pragma unroll
-        for (int e = 0; e < PER; ++e) {
-            const int i = lane + e * WAVE;
-            const bool ok = i < D;
-            fa[e] = ok ? to_f32(pa[((long long)t * Ha + ha) * D + i]) : 0.f;
-            fk[e] = ok ? to_f32(pk[((long long)t * Ha + ha) * D + i]) : 0.f;
-            fw[e] = ok ? p.decay_in[((long long)t * H + head) * D + i] : 0.f;
+            for (int e = 0; e < PER; ++e) {
+                const int ic = min(lane + e * WAVE, D - 1);
+                fa[tt][e] = pa[(t * Ha + ha) * D + ic];
+                fk[tt][e] = pk[(t * Ha + ha) * D + ic];
+                fw[tt][e] = p.decay[(t * H + head) * D + ic];
+            }
+            fv[tt] = pv[(t * H + head) * Dv + jc];
+            fb[tt] = p.scalar[t * H + head];
         }
-        fv = jv ? to_f32(pv[((long long)t * H + head) * Dv + j]) : 0.f;
-        if (DELTA) fb = p.beta_in[(long long)t * H + head];
     };
-    fetch(t0);
-    for (int it = 0; it < n; ++it) {
-        const int t = t0 + it, buf = it & 1;
-        const float v = fv;
-        float beta = 0.f;
-        // stage this token's key-channel vectors
+    // one token: the state's rows of this lane move on and the token's output leaves.  Four partial sums a
+    // lane (rows 0, 1, 2, 3 of every group of four), added in a fixed order, then the quad's exchange.
+    auto token = [&](int tt, float vt, float sc, long long t) {
+        float o4[4] = {0.f, 0.f, 0.f, 0.f};
         if (DELTA) {
-            float qq = 0.f, kk = 0.f;
+            float kv4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int e = 0; e < PER; ++e) { qq = fmaf(fa[e], fa[e], qq); kk = fmaf(fk[e], fk[e], kk); }
-            qq = wave_sum(qq); kk = wave_sum(kk);
-            const float qn = q_scale / sqrtf(qq + 1e-6f), kn = 1.0f / sqrtf(kk + 1e-6f);
-#pragma unroll
-            for (int e = 0; e < PER; ++e) {
-                const int i = lane + e * WAVE;
-                if (i < DP) {
-                    sa[buf][i] = fa[e] * qn;
-                    sk[buf][i] = fk[e] * kn;
-                    sw[buf][i] = i < D ? expf(neg_rate * softplusf_(fw[e] + bias[e])) : 0.f;
-                }
-            }
-            beta = sigmoidf_(fb);
-        } else {
-#pragma unroll
-            for (int e = 0; e < PER; ++e) {
-                const int i = lane + e * WAVE;
-                if (i < DP) {
-                    sa[buf][i] = fa[e];
-                    sk[buf][i] = fk[e];
-                    sw[buf][i] = i < D ? expf(-expf(fw[e] + bias[e])) : 0.f;
-                }
-            }
-        }
-        float bonus = 0.f;
-        if (!DELTA) {
-#pragma unroll
-            for (int e = 0; e < PER; ++e) bonus = fmaf(fa[e] * extra[e], fk[e], bonus);
-            bonus = wave_sum(bonus);
-        }
-        if (it + 1 < n) fetch(t + 1);
-        __syncthreads();                               // one wave: orders the LDS writes before the reads
-        float o = 0.f;
-        if (DELTA) {
-            float kv = 0.f;
-#pragma unroll
-            for (int g4 = 0; g4 < NI; ++g4) {
-                const f32x4 w4 = *(const f32x4*)&sw[buf][g4 * 4];
-                const f32x4 k4 = *(const f32x4*)&sk[buf][g4 * 4];
+            for (int g4 = 0; g4 < NI16; ++g4) {
+                const f32x4 w4 = *(const f32x4*)&sw[tt][row0 + g4 * 4];
+                const f32x4 k4 = *(const f32x4*)&sk[tt][row0 + g4 * 4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     s[g4 * 4 + e] *= w4[e];
-                    kv = fmaf(k4[e], s[g4 * 4 + e], kv);
+                    kv4[e] = fmaf(k4[e], s[g4 * 4 + e], kv4[e]);
                 }
             }
-            const float err = beta * (v - kv);
+            const float err = sc * (vt - group_sum<SPLIT>((kv4[0] + kv4[1]) + (kv4[2] + kv4[3])));
 #pragma unroll
-            for (int g4 = 0; g4 < NI; ++g4) {
-                const f32x4 k4 = *(const f32x4*)&sk[buf][g4 * 4];
-                const f32x4 q4 = *(const f32x4*)&sa[buf][g4 * 4];
+            for (int g4 = 0; g4 < NI16; ++g4) {
+                const f32x4 k4 = *(const f32x4*)&sk[tt][row0 + g4 * 4];
+                const f32x4 q4 = *(const f32x4*)&sa[tt][row0 + g4 * 4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     s[g4 * 4 + e] = fmaf(k4[e], err, s[g4 * 4 + e]);
-                    o = fmaf(q4[e], s[g4 * 4 + e], o);
+                    o4[e] = fmaf(q4[e], s[g4 * 4 + e], o4[e]);
                 }
             }
         } else {
 #pragma unroll
-            for (int g4 = 0; g4 < NI; ++g4) {
-                const f32x4 w4 = *(const f32x4*)&sw[buf][g4 * 4];
-                const f32x4 k4 = *(const f32x4*)&sk[buf][g4 * 4];
-                const f32x4 r4 = *(const f32x4*)&sa[buf][g4 * 4];
+            for (int g4 = 0; g4 < NI16; ++g4) {
+                const f32x4 w4 = *(const f32x4*)&sw[tt][row0 + g4 * 4];
+                const f32x4 k4 = *(const f32x4*)&sk[tt][row0 + g4 * 4];
+                const f32x4 r4 = *(const f32x4*)&sa[tt][row0 + g4 * 4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    o = fmaf(r4[e], s[g4 * 4 + e], o);
-                    s[g4 * 4 + e] = fmaf(w4[e], s[g4 * 4 + e], k4[e] * v);
+                    o4[e] = fmaf(r4[e], s[g4 * 4 + e], o4[e]);
+                    s[g4 * 4 + e] = fmaf(w4[e], s[g4 * 4 + e], k4[e] * vt);
                 }
             }
-            o = fmaf(bonus, v, o);
         }
-        if (jv) p.out[((long long)t * H + head) * Dv + j] = o;
+        float o = group_sum<SPLIT>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+        if (!DELTA) o = fmaf(sc, vt, o);
+        // (the lanes of a group hold the same sum and write it to the same place: no lane is switched off for it)
+        if (jv) p.out[(t * H + head) * Dv + j] = o;
+    };
+
+    fetch(t0, min(n, CH));
+    for (int c0 = 0; c0 < n; c0 += CH) {
+        const int count = min(CH, n - c0);
+        float v[CH], sc[CH];
+#pragma unroll
+        for (int tt = 0; tt < CH; ++tt) {
+            v[tt] = to_f32(fv[tt]);
+            sc[tt] = fb[tt];
+#pragma unroll
+            for (int e = 0; e < PER; ++e) {
+                const int i = lane + e * WAVE;
+                const bool ok = i < D;                 // (tokens beyond the chunk's last are staged and never read)
+                if (i < DP) { sa[tt][i] = ok ? to_f32(fa[tt][e]) : 0.f; sk[tt][i] = ok ? to_f32(fk[tt][e]) : 0.f; sw[tt][i] = ok ? fw[tt][e] : 0.f; }
+            }
+        }
+        if (c0 + CH < n) fetch(t0 + c0 + CH, min(CH, n - c0 - CH));
+        // The workgroup is one wave and LDS serves a wave's accesses in order: nothing has to be waited for
+        // between the writes above and the reads below, only the compiler must keep their order.  (A
+        // __syncthreads() would also wait for the loads of the next eight tokens, which are meant to be under
+        // way while these are computed.)
+        __builtin_amdgcn_wave_barrier();
+        const long long tb = t0 + c0;
+        if (count == CH) {                             // eight whole tokens: no test between them
+#pragma unroll
+            for (int tt = 0; tt < CH; ++tt) token(tt, v[tt], sc[tt], tb + tt);
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < CH; ++tt)
+                if (tt < count) token(tt, v[tt], sc[tt], tb + tt);
+        }
+        __builtin_amdgcn_wave_barrier();               // the reads stay before the next tokens' writes
     }
 #pragma unroll
-    for (int i = 0; i < DP; ++i)
-        if (jv && i < D) S[(long long)i * Dv] = s[i];
+    for (int i = 0; i < RP; ++i)
+        if (jv && row0 + i < D) S[(long long)(row0 + i) * Dv] = s[i];
 }
 
 // ---------------------------------------------------------- per-head unit norm, weight and gate
@@ -279,20 +352,20 @@ __global__ __launch_bounds__(WAVE) void head_norm_gate_kernel(const float* __res
     }
 }
 
-template <typename T, bool DELTA>
+template <typename TA, typename T, bool DELTA>
 int launch_scan(const ScanArgs& p, int R, hipStream_t stream) {
-    const int ni = (p.D + 3) / 4;
-    dim3 grid(R, p.H, ceil_div(p.Dv, WAVE)), block(WAVE);
-#define SCAN(NI) hipLaunchKernelGGL((scan_kernel<T, NI, DELTA>), grid, block, 0, stream, p)
-    if (ni <= 4) SCAN(4);
-    else if (ni <= 8) SCAN(8);
-    else if (ni <= 12) SCAN(12);
-    else if (ni <= 16) SCAN(16);
-    else if (ni <= 24) SCAN(24);
-    else if (ni <= 32) SCAN(32);
-    else if (ni <= 48) SCAN(48);
-    else if (ni <= 64) SCAN(64);
-    else return -2;
+    if (p.H > 65535 || p.D > 256) return -2;
+    const bool narrow = p.D <= 32;                      // four lanes a value channel; else sixteen
+    const int split = narrow ? 4 : 16;
+    const int ni = narrow ? (p.D + 15) / 16 : (p.D + 63) / 64;
+    dim3 grid(R, p.H, ceil_div(p.Dv, WAVE / split)), block(WAVE);
+    if (grid.z > 65535) return -2;
+#define SCAN(NI, SPLIT) hipLaunchKernelGGL((scan_kernel<TA, T, NI, SPLIT, DELTA>), grid, block, 0, stream, p)
+    if (narrow) { if (ni <= 1) SCAN(1, 4); else SCAN(2, 4); }
+    else if (ni <= 1) SCAN(1, 16);
+    else if (ni <= 2) SCAN(2, 16);
+    else if (ni <= 3) SCAN(3, 16);
+    else SCAN(4, 16);
 #undef SCAN
     return launch_status();
 }
@@ -334,27 +407,36 @@ TUFF_EXPORT int tuff_conv_act(const void* x, int dt, const float* taps, float* s
     return launch_status();
 }
 
-// wkv: r, k [T][H*D], v [T][H*D] of type dt; lw float32 [T][H*D]; w0 float32 [H*D]; u float32 [H][D];
-// state float32 [slots][H][D][D]; out float32 [T][H][D].
-TUFF_EXPORT int tuff_wkv_scan(const void* r, const void* k, const void* v, int dt, const float* lw, const float* w0,
-                              const float* u, float* state, float* out, const int* q_start, const int* q_len,
-                              const int* state_slot, int n_requests, int H, int D, hipStream_t stream) {
-    if (n_requests <= 0) return 0;
-    ScanArgs p{r, k, v, lw, w0, u, nullptr, state, out, q_start, q_len, state_slot, H, H, D, D};
-    return dt == DT_F32 ? launch_scan<float, false>(p, n_requests, stream) : launch_scan<bf16_t, false>(p, n_requests, stream);
+// wkv: r, k, v [T][H*D] of type dt; lw float32 [T][H*D] (overwritten with the decays); w0 float32 [H*D]; u float32
+// [H][D]; bonus float32 [T][H] (work array); state float32 [slots][H][D][D]; out float32 [T][H][D].
+TUFF_EXPORT int tuff_wkv_scan(const void* r, const void* k, const void* v, int dt, float* lw, const float* w0,
+                              const float* u, float* bonus, float* state, float* out, const int* q_start, const int* q_len,
+                              const int* state_slot, int n_tokens, int n_requests, int H, int D, hipStream_t stream) {
+    if (n_requests <= 0 || n_tokens <= 0) return 0;
+    if (H > 65535) return -2;
+    PrepArgs pp{r, k, lw, w0, u, nullptr, nullptr, nullptr, bonus, H, H, D};
+    if (dt == DT_F32) hipLaunchKernelGGL((scan_prep_kernel<float, false>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
+    else hipLaunchKernelGGL((scan_prep_kernel<bf16_t, false>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
+    ScanArgs p{r, k, v, lw, bonus, state, out, q_start, q_len, state_slot, H, H, D, D};
+    return dt == DT_F32 ? launch_scan<float, float, false>(p, n_requests, stream)
+                        : launch_scan<bf16_t, bf16_t, false>(p, n_requests, stream);
 }
 
-// delta: q, k [T][Hk*D], v [T][H*Dv] of type dt (after convolution and activation, not yet unit
-// vectors); a float32 [T][H*D]; dt_bias float32 [H*D]; A_log float32 [H]; b float32 [T][H];
-// state float32 [slots][H][D][Dv]; out float32 [T][H][Dv].
-TUFF_EXPORT int tuff_delta_scan(const void* q, const void* k, const void* v, int dt, const float* a, const float* dt_bias,
-                                const float* A_log, const float* b, float* state, float* out, const int* q_start,
-                                const int* q_len, const int* state_slot, int n_requests, int H, int Hk, int D, int Dv,
-                                hipStream_t stream) {
-    if (n_requests <= 0) return 0;
-    if (Hk <= 0 || H % Hk) return -2;
-    ScanArgs p{q, k, v, a, dt_bias, A_log, b, state, out, q_start, q_len, state_slot, H, Hk, D, Dv};
-    return dt == DT_F32 ? launch_scan<float, true>(p, n_requests, stream) : launch_scan<bf16_t, true>(p, n_requests, stream);
+// delta: q, k [T][Hk*D], v [T][H*Dv] of type dt (after convolution and activation, not yet unit vectors); a float32
+// [T][H*D] (overwritten with the decays); dt_bias float32 [H*D]; A_log float32 [H]; b float32 [T][H]; work arrays
+// qn, kn float32 [T][H*D] and beta float32 [T][H]; state float32 [slots][H][D][Dv]; out float32 [T][H][Dv].
+TUFF_EXPORT int tuff_delta_scan(const void* q, const void* k, const void* v, int dt, float* a, const float* dt_bias,
+                                const float* A_log, const float* b, float* qn, float* kn, float* beta, float* state,
+                                float* out, const int* q_start, const int* q_len, const int* state_slot, int n_tokens,
+                                int n_requests, int H, int Hk, int D, int Dv, hipStream_t stream) {
+    if (n_requests <= 0 || n_tokens <= 0) return 0;
+    if (Hk <= 0 || H % Hk || H > 65535) return -2;
+    PrepArgs pp{q, k, a, dt_bias, A_log, b, qn, kn, beta, H, Hk, D};
+    if (dt == DT_F32) hipLaunchKernelGGL((scan_prep_kernel<float, true>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
+    else hipLaunchKernelGGL((scan_prep_kernel<bf16_t, true>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
+    ScanArgs p{qn, kn, v, a, beta, state, out, q_start, q_len, state_slot, H, H, D, Dv};
+    return dt == DT_F32 ? launch_scan<float, float, true>(p, n_requests, stream)
+                        : launch_scan<float, bf16_t, true>(p, n_requests, stream);
 }
 
 // gate_dt: type of the gate's rows (float32 sums of a product may come in as they are); dt: type of y.
