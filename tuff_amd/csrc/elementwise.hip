@@ -226,22 +226,27 @@ __device__ __forceinline__ float activation(float z, int kind) {
 // act[t, f] = f(g) * u with g = gu[t, f], u = gu[t, F + f]: the gated product of a feed-forward whose
 // gate and up rows are stacked, for any of the activations above.
 template <typename TI, typename T>
-__global__ void glu_kernel(const TI* __restrict__ gu, T* __restrict__ act, long long n, int F, int kind) {
+__global__ void glu_kernel(const TI* __restrict__ gu, T* __restrict__ act, long long n, int F, int kind,
+                           const float* __restrict__ bias) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const long long t = i / F;
     const int f = (int)(i - t * F);
-    act[i] = from_f32<T>(activation(to_f32(gu[t * 2 * F + f]), kind) * to_f32(gu[t * 2 * F + F + f]));
+    float g = to_f32(gu[t * 2 * F + f]), u = to_f32(gu[t * 2 * F + F + f]);
+    if (bias) { g += bias[f]; u += bias[F + f]; }
+    act[i] = from_f32<T>(activation(g, kind) * u);
 }
 
-// in_dt: type of gu (float32 sums of a product with its biases may come in as they are); dt: type of act.
-TUFF_EXPORT int tuff_glu(const void* gu, int in_dt, void* act, int dt, int n_tokens, int F, int kind, hipStream_t stream) {
+// in_dt: type of gu (float32 sums of a product may come in as they are); dt: type of act.  bias (float32 [2 F],
+// or null) is added to gu first: the biases of the gate and of the up projection.
+TUFF_EXPORT int tuff_glu(const void* gu, int in_dt, void* act, int dt, int n_tokens, int F, int kind, const float* bias,
+                         hipStream_t stream) {
     const long long n = (long long)n_tokens * F;
     if (n <= 0) return 0;
     dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
-    if (dt == DT_F32 && in_dt == DT_F32) hipLaunchKernelGGL((glu_kernel<float, float>), grid, block, 0, stream, (const float*)gu, (float*)act, n, F, kind);
-    else if (in_dt == DT_F32) hipLaunchKernelGGL((glu_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)gu, (bf16_t*)act, n, F, kind);
-    else if (dt == DT_BF16) hipLaunchKernelGGL((glu_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)act, n, F, kind);
+    if (dt == DT_F32 && in_dt == DT_F32) hipLaunchKernelGGL((glu_kernel<float, float>), grid, block, 0, stream, (const float*)gu, (float*)act, n, F, kind, bias);
+    else if (in_dt == DT_F32) hipLaunchKernelGGL((glu_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)gu, (bf16_t*)act, n, F, kind, bias);
+    else if (dt == DT_BF16) hipLaunchKernelGGL((glu_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)act, n, F, kind, bias);
     else return -2;
     return launch_status();
 }

@@ -36,12 +36,12 @@ _SIGNATURES = {
         "tuff_fill_u32": [_c_void_p, ctypes.c_uint32, _c_ll, _c_void_p],
         "tuff_scatter_i32": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p],
         "tuff_dyt": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
-        "tuff_glu": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_glu": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_act_rows": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
         "tuff_pad_cols": [_c_void_p, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p],
     },
     "recurrent": {
-        "tuff_shift_mix": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+        "tuff_shift_mix": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                            _c_int, _c_int, _c_int, _c_void_p],
         "tuff_shift_state": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
         "tuff_conv_act": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
@@ -50,7 +50,7 @@ _SIGNATURES = {
                           _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_delta_scan": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                             _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                            _c_int, _c_int, _c_int, _c_void_p],
+                            _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_void_p],
         "tuff_head_norm_gate": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int,
                                 _c_float, _c_void_p],
     },
@@ -361,11 +361,13 @@ def dyt(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, alpha: torch.Tensor, 
 ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "relu2": 2, "tanh": 3, "sigmoid": 4}
 
 
-def glu(gu: torch.Tensor, act: torch.Tensor, activation: str) -> None:
-    """act[t, f] = activation(gu[t, f]) * gu[t, F + f]; gu of act's type or float32."""
+def glu(gu: torch.Tensor, act: torch.Tensor, activation: str, bias: Optional[torch.Tensor] = None) -> None:
+    """act[t, f] = activation(gu[t, f] + bias[f]) * (gu[t, F + f] + bias[F + f]); gu of act's type or float32, bias
+    float32 [2 F] or None."""
     n, F = act.shape
     _check(load("elementwise").tuff_glu(
-        _gpu("gu", gu, shape=(n, 2 * F)), _dt(gu), _gpu("act", act), _dt(act), n, F, ACTIVATIONS[activation], _stream()), "glu")
+        _gpu("gu", gu, shape=(n, 2 * F)), _dt(gu), _gpu("act", act), _dt(act), n, F, ACTIVATIONS[activation],
+        _opt("bias", bias, torch.float32, (2 * F,)), _stream()), "glu")
 
 
 def act_rows(inp: torch.Tensor, out: torch.Tensor, activation: str, row_gate: Optional[torch.Tensor] = None,
@@ -1050,17 +1052,19 @@ def shortconv_state(bcx, state, *, q_start, q_len, state_slot, K) -> None:
 
 
 # -------------------------------------------------------------------- recurrent mixers
-def shift_mix(h, prev_state, mu, out, *, req_of_token, q_start, state_slot) -> None:
+def shift_mix(h, prev_state, mu, out, *, req_of_token, q_start, state_slot, q_len=None) -> None:
     """out[s, t] = h[t] + (h[t - 1] - h[t]) * mu[s]; the row before a request's first token of the step is
-    prev_state[slot] (float32 [slots, d]).  h [T, d]; mu float32 [n, d]; out [n, T, d] of h's type."""
+    prev_state[slot] (float32 [slots, d]).  h [T, d]; mu float32 [n, d]; out [n, T, d] of h's type.  With q_len
+    the state is then rewritten with each request's last row of the step (as shift_state does); without, it is
+    only read."""
     T, d = h.shape
     n = mu.shape[0]
     R = q_start.shape[0]
     _check(load("recurrent").tuff_shift_mix(
         _gpu("h", h), _dt(h), _gpu("prev_state", prev_state, torch.float32, (None, d)), _gpu("mu", mu, torch.float32, (n, d)),
         _gpu("out", out, h.dtype, (n, T, d)), _gpu("req_of_token", req_of_token, torch.int32, (T,)),
-        _gpu("q_start", q_start, torch.int32, (R,)), _gpu("state_slot", state_slot, torch.int32, (R,)), T, d, n, _stream()),
-        "shift_mix")
+        _gpu("q_start", q_start, torch.int32, (R,)), _opt("q_len", q_len, torch.int32, (R,)),
+        _gpu("state_slot", state_slot, torch.int32, (R,)), T, d, n, _stream()), "shift_mix")
 
 
 def shift_state(h, prev_state, *, q_start, q_len, state_slot) -> None:
@@ -1127,17 +1131,24 @@ def delta_scan(q, k, v, a, dt_bias, A_log, b, state, out, *, q_start, q_len, sta
     T = q.shape[0]
     R = q_start.shape[0]
     dt = q.dtype
+    # q, k and v may be column ranges of one wider tensor (the convolution's output): rows of one stride
+    ld, ldv = q.stride(0), v.stride(0)
+    for name, t, width, want in (("q", q, Hk * D, ld), ("k", k, Hk * D, ld), ("v", v, H * Dv, ldv)):
+        if (not t.is_cuda or t.dtype != dt or t.dim() != 2 or t.shape != (T, width) or t.stride(1) != 1 or t.stride(0) != want
+                or want < width):
+            raise KernelError(f"delta_scan: {name} must be [{T}, {width}] of {dt} on the GPU with unit column stride (q and k "
+                              f"with one row stride); got {tuple(t.shape)} {t.dtype} stride {t.stride()}")
     if D > SCAN_MAX_DIM or Hk < 1 or H % Hk:
         raise KernelError(f"delta_scan: key size {D} (at most {SCAN_MAX_DIM}) / heads {H}:{Hk} not supported")
     work = torch.empty(2, T, H * D, dtype=torch.float32, device=q.device)       # q and k as unit vectors
     _check(load("recurrent").tuff_delta_scan(
-        _gpu("q", q, shape=(T, Hk * D)), _gpu("k", k, dt, (T, Hk * D)), _gpu("v", v, dt, (T, H * Dv)), _dt(q),
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), _dt(q),
         _gpu("a", a, torch.float32, (T, H * D)), _gpu("dt_bias", dt_bias, torch.float32, (H * D,)),
         _gpu("A_log", A_log, torch.float32, (H,)), _gpu("b", b, torch.float32, (T, H)),
         work[0].data_ptr(), work[1].data_ptr(), torch.empty(T, H, dtype=torch.float32, device=q.device).data_ptr(),
         _gpu("state", state, torch.float32, (None, H, D, Dv)), _gpu("out", out, torch.float32, (T, H * Dv)),
         _gpu("q_start", q_start, torch.int32, (R,)), _gpu("q_len", q_len, torch.int32, (R,)),
-        _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, Hk, D, Dv, _stream()), "delta_scan")
+        _gpu("state_slot", state_slot, torch.int32, (R,)), T, R, H, Hk, D, Dv, ld, ldv, _stream()), "delta_scan")
 
 
 def head_norm_gate(o, w, gate, out, *, H, Dv, eps, per_head_weight: bool, gate_activation: Optional[str]) -> None:

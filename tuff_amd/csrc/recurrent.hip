@@ -22,22 +22,26 @@ __device__ __forceinline__ float softplusf_(float z) { return z > 20.0f ? z : lo
 
 // ------------------------------------------------------------------------ token shift
 // out[s][t][c] = h[t][c] + (prev - h[t][c]) * mu[s][c], prev = the request's token before (its
-// state where t is the first of the step).
+// state where t is the first of the step).  With q_len the workgroup of a request's first token, the only
+// one that reads the request's state, also leaves the state for the next step, the request's last row of
+// this step (each thread after its own read of the same place): no second kernel.
 template <typename T>
-__global__ void shift_mix_kernel(const T* __restrict__ h, const float* __restrict__ prev_state, const float* __restrict__ mu,
+__global__ void shift_mix_kernel(const T* __restrict__ h, float* __restrict__ prev_state, const float* __restrict__ mu,
                                  T* __restrict__ out, const int* __restrict__ req_of_token, const int* __restrict__ q_start,
-                                 const int* __restrict__ state_slot, int n_tokens, int d, int n_mix) {
+                                 const int* __restrict__ q_len, const int* __restrict__ state_slot, int n_tokens, int d, int n_mix) {
     const int t = blockIdx.x;
     const int r = req_of_token[t];
     const bool first = t == q_start[r];
-    const float* ps = prev_state + (long long)state_slot[r] * d;
+    float* ps = prev_state + (long long)state_slot[r] * d;
     const T* hp = h + (long long)(t - 1) * d;
     const T* hc = h + (long long)t * d;
+    const T* hl = (first && q_len) ? h + (long long)(t + q_len[r] - 1) * d : nullptr;
     for (int c = threadIdx.x; c < d; c += blockDim.x) {
         const float x = to_f32(hc[c]);
         const float p = first ? ps[c] : to_f32(hp[c]);
         for (int s = 0; s < n_mix; ++s)
             out[((long long)s * n_tokens + t) * d + c] = from_f32<T>(fmaf(p - x, mu[(long long)s * d + c], x));
+        if (hl) ps[c] = to_f32(hl[c]);
     }
 }
 
@@ -119,7 +123,7 @@ __global__ void conv_state_kernel(const T* __restrict__ x, float* __restrict__ s
 // wkv:    o_j = sum_i r_i S_ij + bonus v_j;   S_ij <- w_i S_ij + k_i v_j
 // delta:  S_ij <- g_i S_ij;  e_j = beta (v_j - sum_i k_i S_ij);  S_ij <- S_ij + k_i e_j;  o_j = sum_i q_i S_ij
 struct PrepArgs {
-    const void *a, *k;              // r or q, k [T][Ha*D] of the compute type
+    const void *a, *k;              // r or q, k: rows of Ha*D of the compute type, lda apart
     float* decay;                   // in: lw or a [T][H*D]; out, in place: w or g
     const float* decay_bias;        // [H*D]: w0 or dt_bias
     const float* per_head;          // wkv: u [H][D];  delta: A_log [H]
@@ -127,6 +131,7 @@ struct PrepArgs {
     float *qn, *kn;                 // delta, out: unit vectors [T][H][D]
     float* scalar;                  // out [T][H]: bonus (wkv) or beta (delta)
     int H, Ha, D;
+    long long lda;                  // elements between two tokens' rows of a and k
 };
 
 template <typename T, bool DELTA>
@@ -135,8 +140,8 @@ __global__ __launch_bounds__(WAVE) void scan_prep_kernel(PrepArgs p) {
     const int head = blockIdx.y, lane = threadIdx.x;
     const int D = p.D, H = p.H, Ha = p.Ha;
     const int ha = head / (H / Ha);
-    const T* pa = (const T*)p.a + (t * Ha + ha) * D;
-    const T* pk = (const T*)p.k + (t * Ha + ha) * D;
+    const T* pa = (const T*)p.a + t * p.lda + ha * D;
+    const T* pk = (const T*)p.k + t * p.lda + ha * D;
     float* dec = p.decay + (t * H + head) * D;
     if (DELTA) {
         float qq = 0.f, kk = 0.f;
@@ -166,13 +171,14 @@ __global__ __launch_bounds__(WAVE) void scan_prep_kernel(PrepArgs p) {
 }
 
 struct ScanArgs {
-    const void *a, *k, *v;          // per token: a (r, or unit q) and k [T][Ha*D], v [T][H*Dv]   (Ha: heads of a and k)
+    const void *a, *k, *v;          // per token: a (r, or unit q) and k [T][Ha*D]; v: rows of H*Dv, ldv apart   (Ha: heads of a and k)
     const float* decay;             // per token [T][H*D]: w or g
     const float* scalar;            // per token [T][H]: bonus or beta
     float* state;                   // [slots][H][D][Dv]
     float* out;                     // [T][H][Dv]
     const int *q_start, *q_len, *state_slot;
     int H, Ha, D, Dv;
+    long long ldv;                  // elements between two tokens' rows of v
 };
 
 constexpr int SCAN_CH = 8;          // tokens staged at a time
@@ -244,7 +250,7 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
                 fk[tt][e] = pk[(t * Ha + ha) * D + ic];
                 fw[tt][e] = p.decay[(t * H + head) * D + ic];
             }
-            fv[tt] = pv[(t * H + head) * Dv + jc];
+            fv[tt] = pv[t * p.ldv + head * Dv + jc];
             fb[tt] = p.scalar[t * H + head];
         }
     };
@@ -371,13 +377,14 @@ int launch_scan(const ScanArgs& p, int R, hipStream_t stream) {
 }
 }  // namespace
 
-TUFF_EXPORT int tuff_shift_mix(const void* h, int dt, const float* prev_state, const float* mu, void* out,
-                               const int* req_of_token, const int* q_start, const int* state_slot,
+// q_len null: the state is only read.
+TUFF_EXPORT int tuff_shift_mix(const void* h, int dt, float* prev_state, const float* mu, void* out,
+                               const int* req_of_token, const int* q_start, const int* q_len, const int* state_slot,
                                int n_tokens, int d, int n_mix, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     dim3 grid(n_tokens), block(256);
-    if (dt == DT_F32) hipLaunchKernelGGL(shift_mix_kernel<float>, grid, block, 0, stream, (const float*)h, prev_state, mu, (float*)out, req_of_token, q_start, state_slot, n_tokens, d, n_mix);
-    else hipLaunchKernelGGL(shift_mix_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)h, prev_state, mu, (bf16_t*)out, req_of_token, q_start, state_slot, n_tokens, d, n_mix);
+    if (dt == DT_F32) hipLaunchKernelGGL(shift_mix_kernel<float>, grid, block, 0, stream, (const float*)h, prev_state, mu, (float*)out, req_of_token, q_start, q_len, state_slot, n_tokens, d, n_mix);
+    else hipLaunchKernelGGL(shift_mix_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)h, prev_state, mu, (bf16_t*)out, req_of_token, q_start, q_len, state_slot, n_tokens, d, n_mix);
     return launch_status();
 }
 
@@ -414,27 +421,28 @@ TUFF_EXPORT int tuff_wkv_scan(const void* r, const void* k, const void* v, int d
                               const int* state_slot, int n_tokens, int n_requests, int H, int D, hipStream_t stream) {
     if (n_requests <= 0 || n_tokens <= 0) return 0;
     if (H > 65535) return -2;
-    PrepArgs pp{r, k, lw, w0, u, nullptr, nullptr, nullptr, bonus, H, H, D};
+    PrepArgs pp{r, k, lw, w0, u, nullptr, nullptr, nullptr, bonus, H, H, D, (long long)H * D};
     if (dt == DT_F32) hipLaunchKernelGGL((scan_prep_kernel<float, false>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
     else hipLaunchKernelGGL((scan_prep_kernel<bf16_t, false>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
-    ScanArgs p{r, k, v, lw, bonus, state, out, q_start, q_len, state_slot, H, H, D, D};
+    ScanArgs p{r, k, v, lw, bonus, state, out, q_start, q_len, state_slot, H, H, D, D, (long long)H * D};
     return dt == DT_F32 ? launch_scan<float, float, false>(p, n_requests, stream)
                         : launch_scan<bf16_t, bf16_t, false>(p, n_requests, stream);
 }
 
-// delta: q, k [T][Hk*D], v [T][H*Dv] of type dt (after convolution and activation, not yet unit vectors); a float32
+// delta: q, k (rows of Hk*D, ld elements apart) and v (rows of H*Dv, ldv apart) of type dt (they
+// may be parts of one wider row), after convolution and activation, not yet unit vectors; a float32
 // [T][H*D] (overwritten with the decays); dt_bias float32 [H*D]; A_log float32 [H]; b float32 [T][H]; work arrays
 // qn, kn float32 [T][H*D] and beta float32 [T][H]; state float32 [slots][H][D][Dv]; out float32 [T][H][Dv].
 TUFF_EXPORT int tuff_delta_scan(const void* q, const void* k, const void* v, int dt, float* a, const float* dt_bias,
                                 const float* A_log, const float* b, float* qn, float* kn, float* beta, float* state,
                                 float* out, const int* q_start, const int* q_len, const int* state_slot, int n_tokens,
-                                int n_requests, int H, int Hk, int D, int Dv, hipStream_t stream) {
+                                int n_requests, int H, int Hk, int D, int Dv, long long ld, long long ldv, hipStream_t stream) {
     if (n_requests <= 0 || n_tokens <= 0) return 0;
     if (Hk <= 0 || H % Hk || H > 65535) return -2;
-    PrepArgs pp{q, k, a, dt_bias, A_log, b, qn, kn, beta, H, Hk, D};
+    PrepArgs pp{q, k, a, dt_bias, A_log, b, qn, kn, beta, H, Hk, D, ld};
     if (dt == DT_F32) hipLaunchKernelGGL((scan_prep_kernel<float, true>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
     else hipLaunchKernelGGL((scan_prep_kernel<bf16_t, true>), dim3(n_tokens, H), dim3(WAVE), 0, stream, pp);
-    ScanArgs p{qn, kn, v, a, beta, state, out, q_start, q_len, state_slot, H, H, D, Dv};
+    ScanArgs p{qn, kn, v, a, beta, state, out, q_start, q_len, state_slot, H, H, D, Dv, ldv};
     return dt == DT_F32 ? launch_scan<float, float, true>(p, n_requests, stream)
                         : launch_scan<float, bf16_t, true>(p, n_requests, stream);
 }

@@ -89,11 +89,12 @@ class GatedMLP(FeedForward):
         self._names = dict(names)
         self._make(self.F)
         self._decls = self.gate_up.weight_decls() + self.down.weight_decls()
+        if self.has_bias:
+            self._decls += [WeightDecl(names["gate.b"], (self.F,), "normal"), WeightDecl(names["up.b"], (self.F,), "normal")]
 
     def _make(self, width: int) -> None:
         n = self._names
-        self.gate_up = Linear([n["gate"], n["up"]], self.d, [width, width],
-                              bias=[n["gate.b"], n["up.b"]] if self.has_bias else None)
+        self.gate_up = Linear([n["gate"], n["up"]], self.d, [width, width])      # (its biases go into the activation's kernel)
         self.down = Linear(n["down"], width, self.d, bias=n["down.b"] if self.has_bias else None)
         self.width = width
 
@@ -120,11 +121,14 @@ class GatedMLP(FeedForward):
             self._make(self.F + pad)
         self.gate_up.bind(weights, rt)
         self.down.bind(weights, rt)
+        self.gu_bias = None
+        if self.has_bias:
+            self.gu_bias = torch.cat([weights[n["gate.b"]].float(), weights[n["up.b"]].float()]).contiguous()
 
     def forward(self, h, ctx, residual, next_norm=None) -> None:
-        gu = self.gate_up.forward(h, out_dtype=torch.float32)       # the activation reads the sums (and biases) as they are
+        gu = self.gate_up.forward(h, out_dtype=torch.float32)       # the activation reads the sums as they are, plus the biases
         act = self.rt.empty(h.shape[0], self.width)
-        ops.glu(gu, act, self.activation)
+        ops.glu(gu, act, self.activation, self.gu_bias)
         self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
 
 

@@ -134,8 +134,8 @@ class WkvMixer(Mixer):
         T, HD = h.shape[0], self.H * self.D
         step = dict(q_start=ctx.q_start, state_slot=ctx.state_slot)
         mixes = self.rt.empty(len(self.MIXES), T, self.d)
-        ops.shift_mix(h, prev.state, self.mu, mixes, req_of_token=ctx.req_of_token, **step)
-        ops.shift_state(h, prev.state, q_len=ctx.q_len, **step)
+        # (the kernel also leaves the state for the next step: each request's last row)
+        ops.shift_mix(h, prev.state, self.mu, mixes, req_of_token=ctx.req_of_token, q_len=ctx.q_len, **step)
         r, k, v = (self.proj[s].forward(mixes[i]) for i, s in enumerate(("r", "k", "v")))
         g = self.proj["g"].forward(mixes[3], out_dtype=torch.float32)          # the gate's activation reads the sums as they are
         lw = self.decay.forward(mixes[4], out_dtype=torch.float32)
@@ -211,8 +211,7 @@ class GatedDeltaMixer(Mixer):
         qkv = self.rt.empty(T, self.C)
         ops.conv_act(x, self.taps, None if tail is None else tail.state, qkv, req_of_token=ctx.req_of_token,
                      q_len=ctx.q_len, activation="silu", **step)
-        # the recurrence reads rows of q, of k and of v: cut apart once (a copy each)
-        q, k, v = (t.contiguous() for t in qkv.split([self.Cq, self.Cq, self.Cv], dim=1))
+        q, k, v = qkv.split([self.Cq, self.Cq, self.Cv], dim=1)         # column ranges of the same rows, no copies
         b = self.beta.forward(h, out_dtype=torch.float32)
         a = self.decay.forward(h, out_dtype=torch.float32)
         gate = self.gate.forward(h, out_dtype=torch.float32)
