@@ -55,21 +55,36 @@ __global__ void route_kernel(const float* __restrict__ z, int stride, int* __res
 // lanes of a wave take every 64th term and add their sums in a fixed butterfly, so a token's logits do not
 // depend on the step it is in), n < N rows of which the first E are experts (the rest: gates of other kinds
 // that are wanted as float32 products of the same rows).
+constexpr int ROUTER_WAVES = 16;
+
 template <typename T>
-__global__ __launch_bounds__(256) void router_kernel(const T* __restrict__ h, const float* __restrict__ W, float* __restrict__ z,
-                                                     int* __restrict__ ids, float* __restrict__ wts, int d, int N, int E,
-                                                     int top, int weight_fn) {
-    extern __shared__ float sm[];
-    float* xs = sm;
-    float* zs = sm + d;
+__global__ __launch_bounds__(ROUTER_WAVES * WAVE) void router_kernel(const T* __restrict__ h, const float* __restrict__ W,
+                                                                      float* __restrict__ z, int* __restrict__ ids,
+                                                                      float* __restrict__ wts, int d, int N, int E, int top,
+                                                                      int weight_fn) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    float* xs = sm;                                        // d floats, padded to a multiple of 4
+    float* zs = sm + ((d + 3) & ~3);
     const long long t = blockIdx.x;
-    for (int c = threadIdx.x; c < d; c += 256) xs[c] = to_f32(h[t * d + c]);
+    for (int c = threadIdx.x; c < d; c += ROUTER_WAVES * WAVE) xs[c] = to_f32(h[t * d + c]);
     __syncthreads();
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    for (int n = wave; n < N; n += 4) {
+    for (int n = wave; n < N; n += ROUTER_WAVES) {
         const float* wr = W + (long long)n * d;
         float acc = 0.f;
-        for (int c = lane; c < d; c += WAVE) acc = fmaf(wr[c], xs[c], acc);
+        if (d % 4 == 0) {
+            // four neighbouring terms a lane and step, several steps' loads under way at a time
+#pragma unroll 8
+            for (int c = lane * 4; c < d; c += 4 * WAVE) {
+                const f32x4 w4 = *(const f32x4*)(wr + c);
+                const f32x4 x4 = *(const f32x4*)(xs + c);
+                acc = fmaf(w4[0], x4[0], acc); acc = fmaf(w4[1], x4[1], acc);
+                acc = fmaf(w4[2], x4[2], acc); acc = fmaf(w4[3], x4[3], acc);
+            }
+        } else {
+#pragma unroll 8
+            for (int c = lane; c < d; c += WAVE) acc = fmaf(wr[c], xs[c], acc);
+        }
         acc = wave_sum(acc);
         if (lane == 0) { zs[n] = acc; z[t * N + n] = acc; }
     }
@@ -284,10 +299,10 @@ TUFF_EXPORT int tuff_moe_experts(const void* h, const void* w_up, const void* w_
 TUFF_EXPORT int tuff_moe_router(const void* h, int dt, const float* W, float* z, int* ids, float* wts, int n_tokens, int d,
                                 int N, int E, int top, int weight_fn, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (top < 1 || top > E || N < E || (long long)(d + N) * 4 > 65536) return -2;
-    const size_t lds = (size_t)(d + N) * sizeof(float);
-    if (dt == DT_F32) hipLaunchKernelGGL(router_kernel<float>, dim3(n_tokens), dim3(256), lds, stream, (const float*)h, W, z, ids, wts, d, N, E, top, weight_fn);
-    else hipLaunchKernelGGL(router_kernel<bf16_t>, dim3(n_tokens), dim3(256), lds, stream, (const bf16_t*)h, W, z, ids, wts, d, N, E, top, weight_fn);
+    if (top < 1 || top > E || N < E || (long long)(d + 4 + N) * 4 > 65536) return -2;
+    const size_t lds = (size_t)(((d + 3) & ~3) + N) * sizeof(float);
+    if (dt == DT_F32) hipLaunchKernelGGL(router_kernel<float>, dim3(n_tokens), dim3(ROUTER_WAVES * WAVE), lds, stream, (const float*)h, W, z, ids, wts, d, N, E, top, weight_fn);
+    else hipLaunchKernelGGL(router_kernel<bf16_t>, dim3(n_tokens), dim3(ROUTER_WAVES * WAVE), lds, stream, (const bf16_t*)h, W, z, ids, wts, d, N, E, top, weight_fn);
     return launch_status();
 }
 

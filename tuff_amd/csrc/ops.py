@@ -1176,7 +1176,7 @@ def moe_route(z, ids, wts, *, E, top, weights: str = "sigmoid") -> None:
                                       {"sigmoid": 0, "softmax": 1}[weights], _stream()), "moe_route")
 
 
-ROUTER_MAX_FLOATS = 16384          # hidden size + logits a token: what the router kernel keeps in LDS
+ROUTER_MAX_FLOATS = 16380          # hidden size + logits a token: what the router kernel keeps in LDS
 
 
 def moe_router(h, w, z, ids, wts, *, E, top, weights: str = "sigmoid") -> None:
