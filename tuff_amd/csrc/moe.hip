@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void grouped_kernel(const bf16_t* __restrict__
         for (int tt = 0; tt < TMT; ++tt) acc[nf][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
     const bf16x8_ zero = {0, 0, 0, 0, 0, 0, 0, 0};
     const bf16_t* We = W + (long long)e * NT16 * KB * 512;
-    constexpr int UN = NF == 1 ? 8 : 2;        // few registers a step: more loads under way (narrow tiles stream the weights)
+    constexpr int UN = NF == 1 ? 8 : 4;        // few registers a step: more loads under way (narrow tiles stream the weights)
 #pragma unroll UN
     for (int kb = 0; kb < KB; ++kb) {
         const int k = kb * 32 + 8 * g;

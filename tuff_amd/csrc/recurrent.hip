@@ -238,25 +238,35 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
     // Every load is issued whatever the lane and token (from a clamped place where there is nothing to fetch);
     // what does not count is replaced when the values are staged, eight tokens later: a load inside a condition
     // would be waited for on the spot, and so would a value that is looked at right after its load.
+    // Addresses are a base that is the same for the whole wave (the chunk's first token, this head) plus a small
+    // offset a lane: the rows of a chunk lie less than 2^31 elements apart.
     const int jc = min(j, Dv - 1);
+    const unsigned strideA = (unsigned)(Ha * D), strideW = (unsigned)(H * D), strideV = (unsigned)p.ldv, strideS = (unsigned)H;
+    int ic[PER];
+#pragma unroll
+    for (int e = 0; e < PER; ++e) ic[e] = min(lane + e * WAVE, D - 1);
     auto fetch = [&](int first, int count) {
+        const TA* ba = pa + ((long long)first * Ha + ha) * D;
+        const TA* bk = pk + ((long long)first * Ha + ha) * D;
+        const float* bw = p.decay + ((long long)first * H + head) * D;
+        const T* bv = pv + (long long)first * p.ldv + (long long)head * Dv;
+        const float* bs = p.scalar + (long long)first * H + head;
 #pragma unroll
         for (int tt = 0; tt < CH; ++tt) {
-            const long long t = first + min(tt, count - 1);
+            const unsigned tc = (unsigned)min(tt, count - 1);
 #pragma unroll
             for (int e = 0; e < PER; ++e) {
-                const int ic = min(lane + e * WAVE, D - 1);
-                fa[tt][e] = pa[(t * Ha + ha) * D + ic];
-                fk[tt][e] = pk[(t * Ha + ha) * D + ic];
-                fw[tt][e] = p.decay[(t * H + head) * D + ic];
+                fa[tt][e] = ba[tc * strideA + (unsigned)ic[e]];
+                fk[tt][e] = bk[tc * strideA + (unsigned)ic[e]];
+                fw[tt][e] = bw[tc * strideW + (unsigned)ic[e]];
             }
-            fv[tt] = pv[t * p.ldv + head * Dv + jc];
-            fb[tt] = p.scalar[t * H + head];
+            fv[tt] = bv[tc * strideV + (unsigned)jc];
+            fb[tt] = bs[tc * strideS];
         }
     };
     // one token: the state's rows of this lane move on and the token's output leaves.  Four partial sums a
     // lane (rows 0, 1, 2, 3 of every group of four), added in a fixed order, then the quad's exchange.
-    auto token = [&](int tt, float vt, float sc, long long t) {
+    auto token = [&](int tt, float vt, float sc, float* orow) {
         float o4[4] = {0.f, 0.f, 0.f, 0.f};
         if (DELTA) {
             float kv4[4] = {0.f, 0.f, 0.f, 0.f};
@@ -297,7 +307,7 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
         float o = group_sum<SPLIT>((o4[0] + o4[1]) + (o4[2] + o4[3]));
         if (!DELTA) o = fmaf(sc, vt, o);
         // (the lanes of a group hold the same sum and write it to the same place: no lane is switched off for it)
-        if (jv) p.out[(t * H + head) * Dv + j] = o;
+        if (jv) orow[(unsigned)tt * (unsigned)(H * Dv)] = o;
     };
 
     fetch(t0, min(n, CH));
@@ -321,14 +331,14 @@ __global__ __launch_bounds__(WAVE) void scan_kernel(ScanArgs p) {
         // __syncthreads() would also wait for the loads of the next eight tokens, which are meant to be under
         // way while these are computed.)
         __builtin_amdgcn_wave_barrier();
-        const long long tb = t0 + c0;
+        float* orow = p.out + ((long long)(t0 + c0) * H + head) * Dv + j;     // this lane's place in the chunk's first row
         if (count == CH) {                             // eight whole tokens: no test between them
 #pragma unroll
-            for (int tt = 0; tt < CH; ++tt) token(tt, v[tt], sc[tt], tb + tt);
+            for (int tt = 0; tt < CH; ++tt) token(tt, v[tt], sc[tt], orow);
         } else {
 #pragma unroll
             for (int tt = 0; tt < CH; ++tt)
-                if (tt < count) token(tt, v[tt], sc[tt], tb + tt);
+                if (tt < count) token(tt, v[tt], sc[tt], orow);
         }
         __builtin_amdgcn_wave_barrier();               // the reads stay before the next tokens' writes
     }
