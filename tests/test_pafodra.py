@@ -22,6 +22,9 @@ def test_registered_by_its_one_name_spelling():
     cfg = cfg_of(pu.P_MIXED)
     assert isinstance(cfg, PafodraConfig) and cfg.vocab_size == 211 and cfg.hidden_size == 64
     assert cfg.owner(3) == 1 and cfg.owner(4) == 0 and cfg.owner(5) == 5
+    chained = copy.deepcopy(pu.P_MIXED)
+    chained["layers"].append(dict(chained["layers"][3], weights_of=3))          # through layer 3 to layer 1
+    assert cfg_of(chained).owner(6) == 1
     assert cfg.rank(0, "w") == 8 and cfg.rank(5, "g") == 20
     again = cfg_of(cfg.to_dict())
     assert again.layers == cfg.layers and again.ranks == cfg.ranks
@@ -34,8 +37,9 @@ def test_registered_by_its_one_name_spelling():
     (lambda r: r["layers"][2]["mixer"].update(conv=0), "conv"),
     (lambda r: r["layers"][1]["mlp"]["router"].update(top=9), "top"),
     (lambda r: r["layers"][3].update(weights_of=3), "weights_of"),
-    (lambda r: r["layers"][3].update(weights_of=4), "weights_of"),
-    (lambda r: r["layers"][3]["mixer"].update(heads=8), "not described"),
+    (lambda r: r["layers"][3].update(weights_of=4), "which is a 'wkv' layer"),
+    (lambda r: r["layers"][3].update(weights_of=0), "layer"),
+    (lambda r: (r["layers"][3].update(weights_of=4), r["layers"][4].update(weights_of=3)), "weights_of"),
     (lambda r: r["norm"].update(eps=0), "eps"),
     (lambda r: r.pop("width"), "width"),
 ])

@@ -85,11 +85,14 @@ class PafodraConfig(ModelConfig):
             if j is not None:
                 if isinstance(j, bool) or not isinstance(j, int) or not 0 <= j < len(self.layers) or j == i:
                     raise ConfigError(f"{where}.weights_of must name another layer, got {j!r}")
-                if self.layers[j].get("weights_of") is not None:
-                    raise ConfigError(f"{where}.weights_of names layer {j}, which has no tensors of its own")
-                src = self.layers[j]
-                if (src.get("type"), src.get("mixer"), src.get("mlp")) != (layer["type"], m, mlp):
-                    raise ConfigError(f"{where} uses the tensors of layer {j} but is not described as that layer is")
+                seen = {i}
+                while self.layers[j].get("weights_of") is not None:          # a layer that itself runs another's tensors
+                    seen.add(j)
+                    j = self.layers[j]["weights_of"]
+                    if isinstance(j, bool) or not isinstance(j, int) or not 0 <= j < len(self.layers) or j in seen:
+                        raise ConfigError(f"{where}.weights_of leads to no layer with tensors of its own")
+                if self.layers[j].get("type") != layer["type"]:
+                    raise ConfigError(f"{where} uses the tensors of layer {j}, which is a '{self.layers[j].get('type')}' layer")
 
     # --------------------------------------------------------------------- derived
     @property
@@ -105,9 +108,10 @@ class PafodraConfig(ModelConfig):
         return float(self.norm["eps"])
 
     def owner(self, i: int) -> int:
-        """The layer whose tensors layer i runs."""
-        j = self.layers[i].get("weights_of")
-        return i if j is None else j
+        """The layer whose tensors layer i runs (its sizes are that layer's)."""
+        while self.layers[i].get("weights_of") is not None:
+            i = self.layers[i]["weights_of"]
+        return i
 
     def rank(self, i: int, which: str) -> int:
         return int(((self.ranks or {}).get(f"l{i}") or {}).get(which, DEFAULT_RANKS[which]))
