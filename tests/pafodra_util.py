@@ -75,6 +75,7 @@ ONLY = {
     "attention": config(48, 101, [layer(attn(4, 2, 16, 8, 0.35))]),
     "attention_equal": config(64, 101, [layer(attn(2, 1, 64, 64, 0.125))]),
     "wkv": config(48, 101, [layer(wkv(2, 24))], ranks={"l0": {"w": 8}}),
+    "wkv_wide": config(48, 101, [layer(wkv(1, 144))], ranks={"l0": {"w": 8}}),          # a head of 144: three quarters of the widest form
     "delta": config(48, 101, [layer(delta(4, 2, 16, 24, 4))], ranks={"l0": {"a": 8, "g": 8}}),
     # one tap: the convolution keeps no tail; the second layer runs the first one's tensors on a state of its own
     "delta_one_tap": config(40, 101, [layer(delta(2, 1, 8, 12, 1)), layer(delta(2, 1, 8, 12, 1), weights_of=0)],

@@ -285,7 +285,7 @@ def test_delta_scan_carries_its_state_across_any_cut(gpu):
     between slots of NaN, float32, against the plain loop."""
     from tuff_amd.csrc import ops
     gen = torch.Generator().manual_seed(5)
-    for H, Hk, D, Dv in [(2, 2, 16, 16), (3, 1, 40, 72), (1, 1, 100, 130)]:
+    for H, Hk, D, Dv in [(2, 2, 16, 16), (3, 1, 40, 72), (1, 1, 100, 130), (2, 1, 200, 24), (1, 1, 256, 8)]:
         n = 23
         rnd = lambda *s: torch.randn(*s, generator=gen)
         q, k, v = rnd(n, Hk * D), rnd(n, Hk * D), rnd(n, H * Dv)
