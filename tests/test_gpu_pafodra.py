@@ -215,7 +215,8 @@ def _sink_softmax(q, k, v, sink, scale):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("dk, dv, H, G", [(16, 16, 4, 2), (64, 64, 8, 2), (24, 40, 3, 1), (128, 128, 2, 2)])
+@pytest.mark.parametrize("dk, dv, H, G", [(16, 16, 4, 2), (64, 64, 8, 2), (24, 40, 3, 1), (128, 128, 2, 2), (256, 256, 2, 1),
+                                          (32, 32, 24, 1)])
 def test_attention_kernels_one_key_stands_out(gpu, dk, dv, H, G, dtype):
     """One key, at the start, far back, at a page's border or the last, is made to hold most of the weight
     beside a sink that holds a known share; the step's queries see it from a prompt's portion and from single
