@@ -57,13 +57,14 @@ class CacheStorage:
             n = manager.groups[gi].pool.num_pages
             shape = (n, spec.num_kv_heads, ps, spec.head_dim)
             vshape = (n, spec.num_kv_heads, ps, spec.v_dim) if spec.value_rows else (n, spec.num_kv_heads, spec.v_dim, ps)
-            if poison:
-                # stale reads show up as NaN in the logits
-                k = torch.full(shape, float("nan"), dtype=dtype, device=device)
-                v = torch.full(vshape, float("nan"), dtype=dtype, device=device)
-            else:
-                k = torch.empty(shape, dtype=dtype, device=device)
-                v = torch.empty(vshape, dtype=dtype, device=device)
+            if spec.values_in_keys:
+                if spec.v_dim > spec.head_dim:
+                    raise ValueError(f"cache entry {e}: values inside the key rows cannot be wider than the keys")
+                vshape = None                    # the key rows are all there is
+            make = (lambda s: torch.full(s, float("nan"), dtype=dtype, device=device)) if poison else \
+                (lambda s: torch.empty(s, dtype=dtype, device=device))        # poison: stale reads show up as NaN in the logits
+            k = make(shape)
+            v = None if vshape is None else make(vshape)
             self.views[e] = PagedKVView(k, v, gi, ps, spec.window)
         for e, spec in layout.states.items():
             # a slot is a whole number of 32-bit words, so that one fill kernel clears any type
@@ -84,7 +85,8 @@ class CacheStorage:
                 if idx is None:
                     idx = torch.tensor(list(pages), dtype=torch.long, device=v.k.device)
                 v.k[idx] = float("nan")
-                v.v[idx] = float("nan")
+                if v.v is not None:
+                    v.v[idx] = float("nan")
 
     def zero_slot(self, slot: int) -> None:
         for v in self.views.values():
@@ -95,7 +97,7 @@ class CacheStorage:
         n = 0
         for v in self.views.values():
             if isinstance(v, PagedKVView):
-                n += (v.k.numel() + v.v.numel()) * v.k.element_size()
+                n += (v.k.numel() + (0 if v.v is None else v.v.numel())) * v.k.element_size()
             else:
                 n += v.raw.numel() * 4
         return n

@@ -17,20 +17,26 @@
 // have a sink: a learned logit whose exponential counts once in the softmax's denominator and
 // that has neither key nor value (it is not scaled).
 //
-// This is the general kernel: any head size up to 256, any page size, float32 or
+// A head may also have a distance slope: slope_h * (pos - key) is taken off the scaled score (from
+// the integer distance, so that far positions lose no bits).  And the values may be the leading vd
+// channels of the key rows themselves (v_in_k: a cache of one latent row a position that serves as key
+// and value; v_cache is then not read).
+//
+// This is the general kernel: any head size up to 640, any page size, float32 or
 // bfloat16 cache.  One wave per (token, head): lanes are keys for q.k, lanes are
 // channels for p.v.
 #include "common.h"
 #include <math.h>
 
 namespace {
-constexpr int MAX_PER_LANE = 4;
+constexpr int MAX_PER_LANE_WIDE = 10;
 
-template <typename T>
+template <typename T, int MAX_PER_LANE>
 __global__ __launch_bounds__(WAVE) void attention_general_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ out,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ req_of_token,
-    const int* __restrict__ positions, int H, int Hkv, int hd, int vd, int page_size, int window, float scale, const float* __restrict__ sinks) {
+    const int* __restrict__ positions, int H, int Hkv, int hd, int vd, int page_size, int window, float scale, const float* __restrict__ sinks,
+    const float* __restrict__ slopes, int v_in_k) {
     __shared__ float qs[MAX_PER_LANE * WAVE];
     __shared__ float ps[WAVE];
     __shared__ long long voff[WAVE];
@@ -40,6 +46,9 @@ __global__ __launch_bounds__(WAVE) void attention_general_kernel(
     const int lo = (window > 0) ? max(0, pos - window + 1) : 0;
     const int* table = block_table + (long long)req_of_token[t] * max_blocks;
     const T* qrow = q + ((long long)t * H + head) * hd;
+    const float slope = slopes ? slopes[head] : 0.f;
+    const T* v_base = v_in_k ? k_cache : v_cache;
+    const long long v_step = v_in_k ? 1 : page_size;          // from a value's channel to the next
     for (int j = lane; j < hd; j += WAVE) qs[j] = to_f32(qrow[j]);
     __syncthreads();
 
@@ -56,11 +65,12 @@ __global__ __launch_bounds__(WAVE) void attention_general_kernel(
         if (valid) {
             const long long page = table[kt / page_size];
             const long long head_base = (page * Hkv + kvh) * page_size;
-            base = head_base * vd + (kt % page_size);     // V: [vd][page_size], this key's column
+            base = v_in_k ? head_base * hd + (long long)(kt % page_size) * hd      // the key's own row
+                          : head_base * vd + (kt % page_size);                     // V: [vd][page_size], this key's column
             const T* krow = k_cache + head_base * hd + (long long)(kt % page_size) * hd;
             float d = 0.f;
             for (int j = 0; j < hd; ++j) d = fmaf(qs[j], to_f32(krow[j]), d);
-            s = d * scale;
+            s = d * scale - slope * (float)(pos - kt);
         }
         const float m_new = fmaxf(m, wave_max(s));
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -77,11 +87,11 @@ __global__ __launch_bounds__(WAVE) void attention_general_kernel(
         for (int jj = 0; jj < n_keys; ++jj) {
             const float pj = ps[jj];
             if (pj == 0.f) continue;                 // masked (below the window) or underflowed
-            const T* vcol = v_cache + voff[jj];
+            const T* vcol = v_base + voff[jj];
 #pragma unroll
             for (int i = 0; i < MAX_PER_LANE; ++i) {
                 const int j = lane + i * WAVE;
-                if (j < vd) acc[i] = fmaf(pj, to_f32(vcol[(long long)j * page_size]), acc[i]);
+                if (j < vd) acc[i] = fmaf(pj, to_f32(vcol[(long long)j * v_step]), acc[i]);
             }
         }
     }
@@ -106,17 +116,17 @@ __global__ __launch_bounds__(WAVE) void attention_general_kernel(
 TUFF_EXPORT int tuff_attention_general(const void* q, const void* k_cache, const void* v_cache, void* out, int dt,
                                        const int* block_table, int max_blocks, const int* req_of_token,
                                        const int* positions, int n_tokens, int H, int Hkv, int hd, int vd, int page_size,
-                                       int window, float scale, const float* sinks, hipStream_t stream) {
+                                       int window, float scale, const float* sinks, const float* slopes, int v_in_k,
+                                       hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (hd > MAX_PER_LANE * WAVE || vd > MAX_PER_LANE * WAVE || vd <= 0 || Hkv <= 0 || H % Hkv != 0) return -2;
+    const int widest = max(hd, vd);
+    if (widest > MAX_PER_LANE_WIDE * WAVE || vd <= 0 || Hkv <= 0 || H % Hkv != 0 || (v_in_k && vd > hd)) return -2;
     dim3 grid(n_tokens, H), block(WAVE);
-    if (dt == DT_F32)
-        hipLaunchKernelGGL(attention_general_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_cache,
-                           (const float*)v_cache, (float*)out, block_table, max_blocks, req_of_token, positions, H, Hkv, hd, vd,
-                           page_size, window, scale, sinks);
-    else
-        hipLaunchKernelGGL(attention_general_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_cache,
-                           (const bf16_t*)v_cache, (bf16_t*)out, block_table, max_blocks, req_of_token, positions, H, Hkv, hd, vd,
-                           page_size, window, scale, sinks);
+#define LAUNCH(T, PL) hipLaunchKernelGGL((attention_general_kernel<T, PL>), grid, block, 0, stream, (const T*)q, (const T*)k_cache, \
+        (const T*)v_cache, (T*)out, block_table, max_blocks, req_of_token, positions, H, Hkv, hd, vd, page_size, window, scale, \
+        sinks, slopes, v_in_k)
+    if (widest <= 4 * WAVE) { if (dt == DT_F32) LAUNCH(float, 4); else LAUNCH(bf16_t, 4); }
+    else { if (dt == DT_F32) LAUNCH(float, MAX_PER_LANE_WIDE); else LAUNCH(bf16_t, MAX_PER_LANE_WIDE); }
+#undef LAUNCH
     return launch_status();
 }

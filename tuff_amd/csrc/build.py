@@ -38,6 +38,8 @@ MODULES = {
     "shortconv": "shortconv.hip",
     "recurrent": "recurrent.hip",
     "moe": "moe.hip",
+    "hyper": "hyper.hip",
+    "latent": "latent.hip",
     "sampling": "sampling.hip",
 }
 

@@ -224,29 +224,36 @@ __device__ __forceinline__ float activation(float z, int kind) {
 }
 
 // act[t, f] = f(g) * u with g = gu[t, f], u = gu[t, F + f]: the gated product of a feed-forward whose
-// gate and up rows are stacked, for any of the activations above.
+// gate and up rows are stacked, for any of the activations above; kind 5 is the clamped form
+// g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).
 template <typename TI, typename T>
 __global__ void glu_kernel(const TI* __restrict__ gu, T* __restrict__ act, long long n, int F, int kind,
-                           const float* __restrict__ bias) {
+                           const float* __restrict__ bias, float limit, float alpha) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const long long t = i / F;
     const int f = (int)(i - t * F);
     float g = to_f32(gu[t * 2 * F + f]), u = to_f32(gu[t * 2 * F + F + f]);
     if (bias) { g += bias[f]; u += bias[F + f]; }
+    if (kind == 5) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        act[i] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+        return;
+    }
     act[i] = from_f32<T>(activation(g, kind) * u);
 }
 
 // in_dt: type of gu (float32 sums of a product may come in as they are); dt: type of act.  bias (float32 [2 F],
 // or null) is added to gu first: the biases of the gate and of the up projection.
 TUFF_EXPORT int tuff_glu(const void* gu, int in_dt, void* act, int dt, int n_tokens, int F, int kind, const float* bias,
-                         hipStream_t stream) {
+                         float limit, float alpha, hipStream_t stream) {
     const long long n = (long long)n_tokens * F;
     if (n <= 0) return 0;
     dim3 grid((unsigned)ceil_div_ll(n, 256)), block(256);
-    if (dt == DT_F32 && in_dt == DT_F32) hipLaunchKernelGGL((glu_kernel<float, float>), grid, block, 0, stream, (const float*)gu, (float*)act, n, F, kind, bias);
-    else if (in_dt == DT_F32) hipLaunchKernelGGL((glu_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)gu, (bf16_t*)act, n, F, kind, bias);
-    else if (dt == DT_BF16) hipLaunchKernelGGL((glu_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)act, n, F, kind, bias);
+    if (dt == DT_F32 && in_dt == DT_F32) hipLaunchKernelGGL((glu_kernel<float, float>), grid, block, 0, stream, (const float*)gu, (float*)act, n, F, kind, bias, limit, alpha);
+    else if (in_dt == DT_F32) hipLaunchKernelGGL((glu_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)gu, (bf16_t*)act, n, F, kind, bias, limit, alpha);
+    else if (dt == DT_BF16) hipLaunchKernelGGL((glu_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)act, n, F, kind, bias, limit, alpha);
     else return -2;
     return launch_status();
 }

@@ -5,7 +5,10 @@
 // renormalised), 1 softmax over the chosen.  Everything here is float32.
 //
 // Experts: y = W_down act(W_up x) with x the token's input, multiplied by the choice's weight before
-// (scale_input) or y after; act: 0 relu squared, 1 silu, 2 gelu (tanh form).  A (token, choice) pair is a
+// (scale_input) or y after; act: 0 relu squared, 1 silu, 2 gelu (tanh form).  Gated experts have two first
+// matrices: y = W_down glu(W_gate x, W_up x) with glu(g, u) = act(g) u for the three above, or, act 3, the
+// clamped form g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).
+// The router may have a bias: z = W h + b.  A (token, choice) pair is a
 // row of the work arrays; the rows of a token are added into the residual stream in the order of
 // its choices, so the sum does not depend on what else is in the step.
 #include "common.h"
@@ -16,6 +19,14 @@ __device__ __forceinline__ float act_fn(float z, int act) {
     if (act == 0) { const float r = fmaxf(z, 0.f); return r * r; }
     if (act == 1) return z / (1.0f + expf(-z));
     return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// What a gated expert makes of its two products (see the head of the file).
+__device__ __forceinline__ float glu_fn(float g, float u, int act, float limit, float alpha) {
+    if (act != 3) return act_fn(g, act) * u;
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
 }
 
 // The `top` largest of row[0..E-1] in the order (value descending, index ascending) and their weights.
@@ -61,7 +72,7 @@ template <typename T>
 __global__ __launch_bounds__(ROUTER_WAVES * WAVE) void router_kernel(const T* __restrict__ h, const float* __restrict__ W,
                                                                       float* __restrict__ z, int* __restrict__ ids,
                                                                       float* __restrict__ wts, int d, int N, int E, int top,
-                                                                      int weight_fn) {
+                                                                      int weight_fn, const float* __restrict__ bias) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     float* xs = sm;                                        // d floats, padded to a multiple of 4
     float* zs = sm + ((d + 3) & ~3);
@@ -86,6 +97,7 @@ __global__ __launch_bounds__(ROUTER_WAVES * WAVE) void router_kernel(const T* __
             for (int c = lane; c < d; c += WAVE) acc = fmaf(wr[c], xs[c], acc);
         }
         acc = wave_sum(acc);
+        if (bias && n < E) acc += bias[n];
         if (lane == 0) { zs[n] = acc; z[t * N + n] = acc; }
     }
     __syncthreads();
@@ -94,11 +106,12 @@ __global__ __launch_bounds__(ROUTER_WAVES * WAVE) void router_kernel(const T* __
 
 constexpr int ROWS_WG = 16;          // output rows a workgroup of four waves computes
 
-// a[row][f] = act(W_up[e][f] . x), x = h[t] (times the choice's weight), rounded to T as the second product takes it
+// a[row][f] = act(W_up[e][f] . x) (gated: glu(W_gate[e][f] . x, W_up[e][f] . x)), x = h[t] (times the choice's weight),
+// rounded to T as the second product takes it
 template <typename T>
 __global__ __launch_bounds__(256) void expert_up_kernel(const T* __restrict__ h, const T* __restrict__ w_up, const int* __restrict__ ids,
                                                         const float* __restrict__ wts, T* __restrict__ a, int d, int F, int top,
-                                                        int act, int scale_input) {
+                                                        int act, int scale_input, int gated, float limit, float alpha) {
     extern __shared__ float xs[];
     const long long row = blockIdx.x;
     const long long t = row / top;
@@ -108,11 +121,19 @@ __global__ __launch_bounds__(256) void expert_up_kernel(const T* __restrict__ h,
     __syncthreads();
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     for (int f = blockIdx.y * ROWS_WG + wave; f < min(F, (int)(blockIdx.y + 1) * ROWS_WG); f += 4) {
-        const T* wr = w_up + ((long long)e * F + f) * d;
+        // gated: the expert's first matrices lie one after the other, gate [F][d] then up [F][d]
+        const T* wr = w_up + ((long long)e * (gated ? 2 * F : F) + f) * d;
         float acc = 0.f;
         for (int c = lane; c < d; c += WAVE) acc = fmaf(to_f32(wr[c]), xs[c], acc);
         acc = wave_sum(acc);
-        if (lane == 0) a[row * F + f] = from_f32<T>(act_fn(acc, act));
+        float res;
+        if (gated) {
+            const T* wu = wr + (long long)F * d;
+            float up = 0.f;
+            for (int c = lane; c < d; c += WAVE) up = fmaf(to_f32(wu[c]), xs[c], up);
+            res = glu_fn(acc, wave_sum(up), act, limit, alpha);
+        } else res = act_fn(acc, act);
+        if (lane == 0) a[row * F + f] = from_f32<T>(res);
     }
 }
 
@@ -196,7 +217,8 @@ template <int NF, int TMT, bool UP>
 __global__ __launch_bounds__(256) void grouped_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                       const int* __restrict__ tiles, const int* __restrict__ sorted,
                                                       const float* __restrict__ wts, bf16_t* __restrict__ A, float* __restrict__ Y,
-                                                      int K, int N, int top, int act, int scale_input) {
+                                                      int K, int N, int top, int act, int scale_input, int gated, float limit,
+                                                      float alpha) {
     const int tile = blockIdx.x;
     const int e = tiles[3 * tile];
     if (e < 0) return;
@@ -252,6 +274,15 @@ __global__ __launch_bounds__(256) void grouped_kernel(const bf16_t* __restrict__
         for (int tt = 0; tt < TMT; ++tt) {
             if (!valid[tt] || ft0 + nf >= NT16) continue;
             const int col = (ft0 + nf) * 16 + 4 * g;
+            if (UP && gated) {
+                // rows 2f and 2f + 1 of the first matrix are feature f's gate and up: a lane holds two features
+#pragma unroll
+                for (int i = 0; i < 4; i += 2)
+                    if (col + i + 1 < N)
+                        A[(long long)(pos0 + tt * 16 + n16) * (N / 2) + (col + i) / 2] =
+                            (bf16_t)glu_fn(acc[nf][tt][i], acc[nf][tt][i + 1], act, limit, alpha);
+                continue;
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 if (col + i >= N) continue;
@@ -270,23 +301,23 @@ TUFF_EXPORT int tuff_moe_route(const float* z, int stride, int* ids, float* wts,
     return launch_status();
 }
 
-// h [T][d], w_up [E][F][d], w_down [E][d][F] of type dt; ids, wts [T][top]; a [T*top][F] (type dt) and
+// h [T][d], w_up [E][F][d] (gated: [E][2 F][d], an expert's gate rows then its up rows), w_down [E][d][F] of type dt; ids, wts [T][top]; a [T*top][F] (type dt) and
 // y [T*top][d] (float32) are work arrays; residual float32 [T][d].
 TUFF_EXPORT int tuff_moe_experts(const void* h, const void* w_up, const void* w_down, int dt, const int* ids, const float* wts,
                                  void* a, float* y, float* residual, int n_tokens, int d, int F, int top, int act,
-                                 int scale_input, hipStream_t stream) {
+                                 int scale_input, int gated, float limit, float alpha, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (d > 16384 || F > 16384) return -2;
     const long long rows = (long long)n_tokens * top;
     dim3 block(256);
     if (dt == DT_F32) {
         hipLaunchKernelGGL(expert_up_kernel<float>, dim3((unsigned)rows, ceil_div(F, ROWS_WG)), block, d * sizeof(float), stream,
-                           (const float*)h, (const float*)w_up, ids, wts, (float*)a, d, F, top, act, scale_input);
+                           (const float*)h, (const float*)w_up, ids, wts, (float*)a, d, F, top, act, scale_input, gated, limit, alpha);
         hipLaunchKernelGGL(expert_down_kernel<float>, dim3((unsigned)rows, ceil_div(d, ROWS_WG)), block, F * sizeof(float), stream,
                            (const float*)a, (const float*)w_down, ids, y, d, F);
     } else {
         hipLaunchKernelGGL(expert_up_kernel<bf16_t>, dim3((unsigned)rows, ceil_div(F, ROWS_WG)), block, d * sizeof(float), stream,
-                           (const bf16_t*)h, (const bf16_t*)w_up, ids, wts, (bf16_t*)a, d, F, top, act, scale_input);
+                           (const bf16_t*)h, (const bf16_t*)w_up, ids, wts, (bf16_t*)a, d, F, top, act, scale_input, gated, limit, alpha);
         hipLaunchKernelGGL(expert_down_kernel<bf16_t>, dim3((unsigned)rows, ceil_div(d, ROWS_WG)), block, F * sizeof(float), stream,
                            (const bf16_t*)a, (const bf16_t*)w_down, ids, y, d, F);
     }
@@ -296,13 +327,14 @@ TUFF_EXPORT int tuff_moe_experts(const void* h, const void* w_up, const void* w_
 }
 
 // z float32 [T][N], the first E columns the experts' logits; ids, wts [T][top].  W float32 [N][d]; h [T][d] of type dt.
+// bias float32 [E] or null: added to the experts' logits before the choice.
 TUFF_EXPORT int tuff_moe_router(const void* h, int dt, const float* W, float* z, int* ids, float* wts, int n_tokens, int d,
-                                int N, int E, int top, int weight_fn, hipStream_t stream) {
+                                int N, int E, int top, int weight_fn, const float* bias, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (top < 1 || top > E || N < E || (long long)(d + 4 + N) * 4 > 65536) return -2;
     const size_t lds = (size_t)(((d + 3) & ~3) + N) * sizeof(float);
-    if (dt == DT_F32) hipLaunchKernelGGL(router_kernel<float>, dim3(n_tokens), dim3(ROUTER_WAVES * WAVE), lds, stream, (const float*)h, W, z, ids, wts, d, N, E, top, weight_fn);
-    else hipLaunchKernelGGL(router_kernel<bf16_t>, dim3(n_tokens), dim3(ROUTER_WAVES * WAVE), lds, stream, (const bf16_t*)h, W, z, ids, wts, d, N, E, top, weight_fn);
+    if (dt == DT_F32) hipLaunchKernelGGL(router_kernel<float>, dim3(n_tokens), dim3(ROUTER_WAVES * WAVE), lds, stream, (const float*)h, W, z, ids, wts, d, N, E, top, weight_fn, bias);
+    else hipLaunchKernelGGL(router_kernel<bf16_t>, dim3(n_tokens), dim3(ROUTER_WAVES * WAVE), lds, stream, (const bf16_t*)h, W, z, ids, wts, d, N, E, top, weight_fn, bias);
     return launch_status();
 }
 
@@ -312,10 +344,12 @@ TUFF_EXPORT int tuff_moe_grouped_tile_rows(long long R, int E) { return R >= 24l
 // The experts of many rows on the matrix cores (bfloat16): h [T][d]; w_up, w_down every expert's matrix in blocks
 // (see grouped_kernel), [E][F x d] and [E][d x F]; ids, wts [T][top]; work arrays sorted int32 [T*top], tiles int32
 // [3 * max_tiles] with max_tiles >= ceil(T*top / tile rows) + E, a bfloat16 [T*top][F], y float32 [T*top][d];
-// residual float32 [T][d].  d and F multiples of 8, E at most 1024.
+// residual float32 [T][d].  d and F multiples of 8, E at most 1024.  gated: w_up is [E][2 F x d] with row 2 f feature
+// f's gate row and row 2 f + 1 its up row.
 TUFF_EXPORT int tuff_moe_experts_grouped(const void* h, const void* w_up, const void* w_down, const int* ids, const float* wts,
                                          int* sorted, int* tiles, int max_tiles, void* a, float* y, float* residual,
-                                         int n_tokens, int d, int F, int E, int top, int act, int scale_input, hipStream_t stream) {
+                                         int n_tokens, int d, int F, int E, int top, int act, int scale_input, int gated,
+                                         float limit, float alpha, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     const long long R = (long long)n_tokens * top;
     if (d % 8 || F % 8 || E > GROUP_MAX_E || E < 1 || R > 0x7fffffffll) return -2;
@@ -324,17 +358,18 @@ TUFF_EXPORT int tuff_moe_experts_grouped(const void* h, const void* w_up, const 
     hipLaunchKernelGGL(group_rows_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)R, E, TM, sorted, tiles, max_tiles);
     const bf16_t* H_ = (const bf16_t*)h;
     bf16_t* A_ = (bf16_t*)a;
+    const int F1 = gated ? 2 * F : F;        // rows of the first matrix (gated: gate and up rows take turns)
     // few rows an expert: many narrow workgroups stream the weights; many: wide ones reuse them
     if (TM == 32) {
-        hipLaunchKernelGGL((grouped_kernel<4, 2, true>), dim3(max_tiles, ceil_div(ceil_div(F, 16), 16)), dim3(256), 0, stream,
-                           H_, (const bf16_t*)w_up, tiles, sorted, wts, A_, nullptr, d, F, top, act, scale_input);
+        hipLaunchKernelGGL((grouped_kernel<4, 2, true>), dim3(max_tiles, ceil_div(ceil_div(F1, 16), 16)), dim3(256), 0, stream,
+                           H_, (const bf16_t*)w_up, tiles, sorted, wts, A_, nullptr, d, F1, top, act, scale_input, gated, limit, alpha);
         hipLaunchKernelGGL((grouped_kernel<4, 2, false>), dim3(max_tiles, ceil_div(ceil_div(d, 16), 16)), dim3(256), 0, stream,
-                           A_, (const bf16_t*)w_down, tiles, sorted, wts, nullptr, y, F, d, top, act, scale_input);
+                           A_, (const bf16_t*)w_down, tiles, sorted, wts, nullptr, y, F, d, top, act, scale_input, 0, 0.f, 0.f);
     } else {
-        hipLaunchKernelGGL((grouped_kernel<1, 1, true>), dim3(max_tiles, ceil_div(ceil_div(F, 16), 4)), dim3(256), 0, stream,
-                           H_, (const bf16_t*)w_up, tiles, sorted, wts, A_, nullptr, d, F, top, act, scale_input);
+        hipLaunchKernelGGL((grouped_kernel<1, 1, true>), dim3(max_tiles, ceil_div(ceil_div(F1, 16), 4)), dim3(256), 0, stream,
+                           H_, (const bf16_t*)w_up, tiles, sorted, wts, A_, nullptr, d, F1, top, act, scale_input, gated, limit, alpha);
         hipLaunchKernelGGL((grouped_kernel<1, 1, false>), dim3(max_tiles, ceil_div(ceil_div(d, 16), 4)), dim3(256), 0, stream,
-                           A_, (const bf16_t*)w_down, tiles, sorted, wts, nullptr, y, F, d, top, act, scale_input);
+                           A_, (const bf16_t*)w_down, tiles, sorted, wts, nullptr, y, F, d, top, act, scale_input, 0, 0.f, 0.f);
     }
     const long long n = (long long)n_tokens * d;
     hipLaunchKernelGGL(combine_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, y, wts, residual, n, d, top, !scale_input);

@@ -36,7 +36,7 @@ _SIGNATURES = {
         "tuff_fill_u32": [_c_void_p, ctypes.c_uint32, _c_ll, _c_void_p],
         "tuff_scatter_i32": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p],
         "tuff_dyt": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
-        "tuff_glu": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
+        "tuff_glu": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_float, _c_float, _c_void_p],
         "tuff_act_rows": [_c_void_p, _c_int, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
         "tuff_pad_cols": [_c_void_p, _c_void_p, _c_int, _c_ll, _c_int, _c_int, _c_void_p],
     },
@@ -57,12 +57,12 @@ _SIGNATURES = {
     "moe": {
         "tuff_moe_route": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_moe_router": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                            _c_int, _c_void_p],
+                            _c_int, _c_void_p, _c_void_p],
         "tuff_moe_grouped_tile_rows": [_c_ll, _c_int],
         "tuff_moe_experts_grouped": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
-                                     _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                     _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
         "tuff_moe_experts": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
     },
     "gemm_f32": {
         "tuff_gemm_f32": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -87,7 +87,7 @@ _SIGNATURES = {
         "tuff_qkv_post": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                           _c_void_p, _c_void_p, _c_int, _c_float,
                           _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
-                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
         "tuff_rope_table": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p],
         "tuff_kv_write": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -95,7 +95,17 @@ _SIGNATURES = {
     "attention": {
         "tuff_attention_general": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
                                    _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                   _c_float, _c_void_p, _c_void_p],
+                                   _c_float, _c_void_p, _c_void_p, _c_int, _c_void_p],
+    },
+    "hyper": {
+        "tuff_hc_step": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                         _c_int, _c_int, _c_int, _c_float, _c_void_p],
+    },
+    "latent": {
+        "tuff_latent_post": [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_float,
+                             _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_head_matmul": [_c_void_p, _c_ll, _c_ll, _c_void_p, _c_void_p, _c_ll, _c_ll, _c_void_p, _c_ll, _c_int,
+                             _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "attention_mfma": {
         "tuff_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -359,15 +369,20 @@ def dyt(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, alpha: torch.Tensor, 
 
 
 ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "relu2": 2, "tanh": 3, "sigmoid": 4}
+GLU_ACTIVATIONS = dict(ACTIVATIONS, swish_clamp=5)
 
 
-def glu(gu: torch.Tensor, act: torch.Tensor, activation: str, bias: Optional[torch.Tensor] = None) -> None:
+def glu(gu: torch.Tensor, act: torch.Tensor, activation: str, bias: Optional[torch.Tensor] = None, *,
+        limit: float = 0.0, alpha: float = 1.0) -> None:
     """act[t, f] = activation(gu[t, f] + bias[f]) * (gu[t, F + f] + bias[F + f]); gu of act's type or float32, bias
-    float32 [2 F] or None."""
+    float32 [2 F] or None.  activation "swish_clamp": g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit),
+    u' = clamp(u, -limit, limit)."""
     n, F = act.shape
+    if activation == "swish_clamp" and not limit > 0:
+        raise KernelError("glu: the clamped form needs a positive limit")
     _check(load("elementwise").tuff_glu(
-        _gpu("gu", gu, shape=(n, 2 * F)), _dt(gu), _gpu("act", act), _dt(act), n, F, ACTIVATIONS[activation],
-        _opt("bias", bias, torch.float32, (2 * F,)), _stream()), "glu")
+        _gpu("gu", gu, shape=(n, 2 * F)), _dt(gu), _gpu("act", act), _dt(act), n, F, GLU_ACTIVATIONS[activation],
+        _opt("bias", bias, torch.float32, (2 * F,)), float(limit), float(alpha), _stream()), "glu")
 
 
 def act_rows(inp: torch.Tensor, out: torch.Tensor, activation: str, row_gate: Optional[torch.Tensor] = None,
@@ -694,10 +709,17 @@ def _gemm_workspace(M: int, N: int, K: int, device, emit: bool = False) -> Optio
 # ----------------------------------------------------------------- q/k/v post-processing
 def qkv_post(qkv, q_out, *, H, Hkv, hd, positions, eps=0.0, q_norm_w=None, k_norm_w=None,
              inv_freq=None, rotary_dim=0, interleaved=False, k_out=None,
-             k_cache=None, v_cache=None, slot_mapping=None, page_size=1, angles=None) -> None:
+             k_cache=None, v_cache=None, slot_mapping=None, page_size=1, angles=None, wide_rows: bool = False) -> None:
+    """wide_rows: a row of qkv holds more than (H + 2 Hkv) hd elements or fewer (values of another width behind the
+    keys); then only q_out and k_out are written (no cache)."""
     T = qkv.shape[0]
     dt = qkv.dtype
-    _gpu("qkv", qkv, shape=(T, (H + 2 * Hkv) * hd))
+    if wide_rows:
+        _gpu("qkv", qkv, shape=(T, None))
+        if qkv.shape[1] < (H + Hkv) * hd or k_cache is not None:
+            raise KernelError("qkv_post: wide rows hold at least the q and k heads and go with no cache write")
+    else:
+        _gpu("qkv", qkv, shape=(T, (H + 2 * Hkv) * hd))
     _gpu("q_out", q_out, dt, (T, H * hd))
     _opt("k_out", k_out, dt, (T, Hkv * hd))
     if (k_cache is None) != (v_cache is None):
@@ -729,7 +751,8 @@ def qkv_post(qkv, q_out, *, H, Hkv, hd, positions, eps=0.0, q_norm_w=None, k_nor
         qkv.data_ptr(), q_out.data_ptr(), p(k_out), p(k_cache), p(v_cache), _dt(qkv),
         p(q_norm_w), p(k_norm_w), norm_dt, float(eps), p(inv_freq), int(rotary_dim), int(interleaved),
         positions.data_ptr(), p(slot_mapping), T, H, Hkv, hd, page_size,
-        p(angles) if inv_freq is not None else None, 0 if angles is None else angles.shape[0], _stream()), "qkv_post")
+        p(angles) if inv_freq is not None else None, 0 if angles is None else angles.shape[0],
+        qkv.shape[1] if wide_rows else 0, _stream()), "qkv_post")
 
 
 def rope_table(inv_freq: torch.Tensor, n_pos: int) -> torch.Tensor:
@@ -760,9 +783,10 @@ def kv_write(k, v, k_cache, v_cache, slot_mapping, *, Hkv, hd, page_size, vd=Non
 
 # -------------------------------------------------------------------------- attention
 def attention_general(q, k_cache, v_cache, out, *, block_table, req_of_token, positions,
-                      H, Hkv, hd, page_size, window=0, scale=None, vd=None, sinks=None) -> None:
+                      H, Hkv, hd, page_size, window=0, scale=None, vd=None, sinks=None, slopes=None) -> None:
     """vd: width of a value where it is not the keys'.  sinks: float32 [H], a logit per head that counts
-    once in the softmax's denominator and has no value."""
+    once in the softmax's denominator and has no value.  slopes: float32 [H]; slopes[h] * (position - key) is
+    taken off head h's scaled scores.  v_cache None: the values are the first vd channels of the key rows."""
     T = q.shape[0]
     dt = q.dtype
     vd = hd if vd is None else int(vd)
@@ -770,22 +794,123 @@ def attention_general(q, k_cache, v_cache, out, *, block_table, req_of_token, po
     _gpu("out", out, dt, (T, H * vd))
     P = k_cache.shape[0]
     _gpu("k_cache", k_cache, dt, (P, Hkv, page_size, hd))
-    _gpu("v_cache", v_cache, dt, (P, Hkv, vd, page_size))
+    if v_cache is None:
+        if vd > hd:
+            raise KernelError("attention: values inside the key rows cannot be wider than the keys")
+    else:
+        _gpu("v_cache", v_cache, dt, (P, Hkv, vd, page_size))
     _opt("sinks", sinks, torch.float32, (H,))
+    _opt("slopes", slopes, torch.float32, (H,))
     _gpu("block_table", block_table, torch.int32)
     if block_table.dim() != 2:
         raise KernelError("attention: block_table must be [requests, blocks]")
     _gpu("req_of_token", req_of_token, torch.int32, (T,))
     _gpu("positions", positions, torch.int32, (T,))
-    if hd > 256 or vd > 256 or H % Hkv:
+    if hd > ATTN_GENERAL_MAX_DIM or vd > ATTN_GENERAL_MAX_DIM or H % Hkv:
         raise KernelError(f"attention: head size {hd} (values {vd}) / heads {H}:{Hkv} not supported")
     if scale is None:
         scale = 1.0 / math.sqrt(hd)
     _check(load("attention").tuff_attention_general(
-        q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _dt(q),
+        q.data_ptr(), k_cache.data_ptr(), None if v_cache is None else v_cache.data_ptr(), out.data_ptr(), _dt(q),
         block_table.data_ptr(), block_table.shape[1], req_of_token.data_ptr(), positions.data_ptr(),
         T, H, Hkv, hd, vd, page_size, int(window or 0), float(scale), None if sinks is None else sinks.data_ptr(),
-        _stream()), "attention_general")
+        None if slopes is None else slopes.data_ptr(), int(v_cache is None), _stream()), "attention_general")
+
+
+ATTN_GENERAL_MAX_DIM = 640   # widest key or value row of the general attention kernel
+
+
+# ------------------------------------------------------------- several residual streams
+HC_MAX_STREAMS, HC_MAX_DIM = 8, 15360
+
+
+def hc_step(xs, *, y=None, mix=None, out_w=None, in_w=None, norm_w=None, eps: float = 0.0, h_out=None, u_out=None) -> None:
+    """One kernel over the residual streams xs (float32 [S, T, d], in place).  With y [T, d], mix [S, S] (indexed
+    [from, to]) and out_w [S]: xs[r] <- sum_s mix[s, r] xs[s] + out_w[r] y.  Then, with in_w [S]: u = sum_s in_w[s]
+    xs[s] (of the new values); with norm_w (float32 [d]) h_out [T, d] = u / sqrt(mean(u^2) + eps) * norm_w in h_out's
+    type, without it u_out [T, d] = u in float32."""
+    S, T, d = xs.shape
+    _gpu("xs", xs, torch.float32)
+    if S > HC_MAX_STREAMS or d > HC_MAX_DIM:
+        raise KernelError(f"hc_step: at most {HC_MAX_STREAMS} streams of at most {HC_MAX_DIM} channels")
+    if (y is None) != (mix is None) or (y is None) != (out_w is None):
+        raise KernelError("hc_step: y, mix and out_w go together")
+    _opt("y", y, torch.float32, (T, d))
+    _opt("mix", mix, torch.float32, (S, S))
+    _opt("out_w", out_w, torch.float32, (S,))
+    _opt("in_w", in_w, torch.float32, (S,))
+    _opt("norm_w", norm_w, torch.float32, (d,))
+    if in_w is not None:
+        if norm_w is not None:
+            _gpu("h_out", h_out, shape=(T, d))
+        else:
+            _gpu("u_out", u_out, torch.float32, (T, d))
+    p = lambda t: None if t is None else t.data_ptr()
+    _check(load("hyper").tuff_hc_step(xs.data_ptr(), p(y), p(mix), p(out_w), p(in_w), p(norm_w), p(h_out),
+                                      DT_F32 if h_out is None else _dt(h_out), p(u_out), S, T, d, float(eps), _stream()), "hc_step")
+
+
+# ------------------------------------------------------------------- latent attention
+def latent_post(proj, q_lat, cache, *, q_off: int, ckr_off: int, norm_w, eps: float, inv_freq, rot_dims: int, positions,
+                slot_mapping, H: int, dim: int, rot: int, rank: int) -> None:
+    """From a token's projected row proj[t] (queries [H, dim + rot] from column q_off; the latent's raw channels
+    [rank] and the shared key part [rot] from column ckr_off): the cache row [norm(c) * norm_w | rotate(k)] at
+    slot_mapping[t] (cache [pages, 1, page size, rank + rot]; slot_mapping None: no write) and the rotated query
+    parts into q_lat[t, h, rank:] (q_lat [T, H * (rank + rot)]).  Rotation of neighbouring pairs of the first rot_dims
+    channels by position * inv_freq (float32 [rot_dims / 2])."""
+    T = proj.shape[0]
+    dt = proj.dtype
+    lat = rank + rot
+    _gpu("proj", proj, shape=(T, None))
+    if q_off + H * (dim + rot) > proj.shape[1] or ckr_off + lat > proj.shape[1] or min(q_off, ckr_off) < 0:
+        raise KernelError("latent_post: the columns lie outside the projected row")
+    _gpu("q_lat", q_lat, dt, (T, H * lat))
+    if cache.dim() != 4 or cache.shape[1] != 1 or cache.shape[3] != lat:
+        raise KernelError(f"latent_post: the cache must be [pages, 1, page size, {lat}], got {tuple(cache.shape)}")
+    _gpu("cache", cache, dt)
+    _gpu("norm_w", norm_w, shape=(rank,))
+    if rot_dims % 2 or not 0 <= rot_dims <= rot:
+        raise KernelError(f"latent_post: {rot_dims} rotated channels of {rot}")
+    if rot_dims:
+        _gpu("inv_freq", inv_freq, torch.float32, (rot_dims // 2,))
+    _gpu("positions", positions, torch.int32, (T,))
+    _opt("slot_mapping", slot_mapping, torch.int32, (T,))
+    _check(load("latent").tuff_latent_post(
+        proj.data_ptr(), proj.shape[1], int(q_off), int(ckr_off), q_lat.data_ptr(), cache.data_ptr(), _dt(proj),
+        norm_w.data_ptr(), _dt(norm_w), float(eps), inv_freq.data_ptr() if rot_dims else None, int(rot_dims),
+        positions.data_ptr(), None if slot_mapping is None else slot_mapping.data_ptr(), T, H, dim, rot, rank, _stream()),
+        "latent_post")
+
+
+HEAD_MATMUL_MAX_K = 2048
+
+
+def head_matmul(x, w, y, *, H: int, x_col: int = 0, x_head: int, y_col: int = 0, y_head: int, gate=None, gate_col: int = 0) -> None:
+    """y[t, y_col + h * y_head + n] = sum_k x[t, x_col + h * x_head + k] * w[h, k, n], n < N, k < K, for w [H, K, N];
+    with gate ([T, *], its column gate_col + h the head's) times sigmoid(gate).  x, w, y, gate of one type; rows of x, y
+    and gate may be wider than what is read or written."""
+    T = x.shape[0]
+    dt = x.dtype
+    Hw, K, N = w.shape
+    _gpu("x", x, shape=(T, None))
+    _gpu("w", w, dt)
+    _gpu("y", y, dt, (T, None))
+    if Hw != H or K > HEAD_MATMUL_MAX_K:
+        raise KernelError(f"head_matmul: w is {tuple(w.shape)} for {H} heads (inner size at most {HEAD_MATMUL_MAX_K})")
+    if x_col + (H - 1) * x_head + K > x.shape[1] or y_col + (H - 1) * y_head + N > y.shape[1] or min(x_col, y_col) < 0:
+        raise KernelError("head_matmul: the heads' columns lie outside a row")
+    if x_head < 0 or (y_head < N and H > 1):
+        raise KernelError("head_matmul: the heads' outputs overlap")
+    gp = None
+    if gate is not None:
+        _gpu("gate", gate, dt, (T, None))
+        if gate_col < 0 or gate_col + H > gate.shape[1]:
+            raise KernelError("head_matmul: the gates' columns lie outside a row")
+        gp = gate.data_ptr() + gate_col * gate.element_size()
+    es = x.element_size()
+    _check(load("latent").tuff_head_matmul(
+        x.data_ptr() + x_col * es, x.shape[1], int(x_head), w.data_ptr(), y.data_ptr() + y_col * es, y.shape[1], int(y_head),
+        gp, 0 if gate is None else gate.shape[1], _dt(x), T, H, K, N, _stream()), "head_matmul")
 
 
 ATTN_PARTITION = 256        # keys a partition of the matrix-core attention kernel covers
@@ -1179,16 +1304,17 @@ def moe_route(z, ids, wts, *, E, top, weights: str = "sigmoid") -> None:
 ROUTER_MAX_FLOATS = 16380          # hidden size + logits a token: what the router kernel keeps in LDS
 
 
-def moe_router(h, w, z, ids, wts, *, E, top, weights: str = "sigmoid") -> None:
+def moe_router(h, w, z, ids, wts, *, E, top, weights: str = "sigmoid", bias=None) -> None:
     """z = h @ w.T in float32 (h [T, d] of the compute type, w float32 [N, d], z float32 [T, N]) and, of its first
-    E columns, the choice as moe_route makes it, in one kernel."""
+    E columns, the choice as moe_route makes it, in one kernel.  bias: float32 [E], added to the experts' logits."""
     T, d = h.shape
     N = w.shape[0]
     if d + N > ROUTER_MAX_FLOATS:
         raise KernelError(f"moe_router: hidden size {d} + {N} logits above {ROUTER_MAX_FLOATS}")
     _check(load("moe").tuff_moe_router(_gpu("h", h), _dt(h), _gpu("w", w, torch.float32, (N, d)), _gpu("z", z, torch.float32, (T, N)),
                                        _gpu("ids", ids, torch.int32, (T, top)), _gpu("wts", wts, torch.float32, (T, top)),
-                                       T, d, N, E, top, {"sigmoid": 0, "softmax": 1}[weights], _stream()), "moe_router")
+                                       T, d, N, E, top, {"sigmoid": 0, "softmax": 1}[weights],
+                                       _opt("bias", bias, torch.float32, (E,)), _stream()), "moe_router")
 
 
 def tile_experts(ws) -> torch.Tensor:
@@ -1200,16 +1326,32 @@ def moe_grouped_supported(dtype, d: int, F: int, E: int) -> bool:
     return dtype == torch.bfloat16 and d % 8 == 0 and F % 8 == 0 and 1 <= E <= 1024
 
 
+EXPERT_ACTIVATIONS = {"relu2": 0, "silu": 1, "gelu_tanh": 2, "swish_clamp": 3}
+
+
+def _expert_activation(activation: str, gated: bool, limit: float) -> int:
+    if activation == "swish_clamp" and (not gated or not limit > 0):
+        raise KernelError("experts: the clamped form needs gated experts and a positive limit")
+    return EXPERT_ACTIVATIONS[activation]
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """[2 F, d] with row 2 f = gate[f] and row 2 f + 1 = up[f]: the first matrix of a gated expert as
+    moe_experts_grouped takes it (before tile_experts)."""
+    return torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
+
+
 def moe_experts_grouped(h, up_tiles, down_tiles, ids, wts, residual, *, F: int, activation: str = "relu2",
-                        scale_input: bool = True) -> None:
+                        scale_input: bool = True, gated: bool = False, limit: float = 0.0, alpha: float = 1.0) -> None:
     """moe_experts on the matrix cores, bfloat16: the rows (token, choice) are sorted by expert and every expert's
-    rows go through its two matrices in tiles.  up_tiles, down_tiles: tile_experts() of the [F, d] and [d, F] matrices."""
+    rows go through its two matrices in tiles.  up_tiles, down_tiles: tile_experts() of the [F, d] and [d, F] matrices;
+    gated: of interleave_gate_up(gate, up) [2 F, d] and [d, F]."""
     T, d = h.shape
     E, top = up_tiles.shape[0], ids.shape[1]
     if not moe_grouped_supported(h.dtype, d, F, E):
         raise KernelError(f"moe_experts_grouped: bfloat16, sizes that are multiples of 8 and at most 1024 experts; got {h.dtype}, {d}, {F}, {E}")
     _gpu("h", h, torch.bfloat16)
-    _gpu("up_tiles", up_tiles, torch.bfloat16, (E, -(-F // 16), -(-d // 32), 64, 8))
+    _gpu("up_tiles", up_tiles, torch.bfloat16, (E, -(-(2 * F if gated else F) // 16), -(-d // 32), 64, 8))
     _gpu("down_tiles", down_tiles, torch.bfloat16, (E, -(-d // 16), -(-F // 32), 64, 8))
     _gpu("ids", ids, torch.int32, (T, top))
     _gpu("wts", wts, torch.float32, (T, top))
@@ -1225,19 +1367,26 @@ def moe_experts_grouped(h, up_tiles, down_tiles, ids, wts, residual, *, F: int, 
     _check(lib.tuff_moe_experts_grouped(h.data_ptr(), up_tiles.data_ptr(), down_tiles.data_ptr(), ids.data_ptr(), wts.data_ptr(),
                                         srt.data_ptr(), tiles.data_ptr(), max_tiles, a.data_ptr(), y.data_ptr(),
                                         residual.data_ptr(), T, d, F, E, top,
-                                        {"relu2": 0, "silu": 1, "gelu_tanh": 2}[activation], int(scale_input), _stream()),
+                                        _expert_activation(activation, gated, limit), int(scale_input), int(gated),
+                                        float(limit), float(alpha), _stream()),
            "moe_experts_grouped")
 
 
-def moe_experts(h, w_up, w_down, ids, wts, residual, *, activation: str = "relu2", scale_input: bool = True) -> None:
+def moe_experts(h, w_up, w_down, ids, wts, residual, *, activation: str = "relu2", scale_input: bool = True,
+                gated: bool = False, limit: float = 0.0, alpha: float = 1.0) -> None:
     """residual[t] += sum over the token's choices of W_down[e] act(W_up[e] x), x = h[t] times the choice's
-    weight (scale_input) or the product times it.  h [T, d]; w_up [E, F, d]; w_down [E, d, F], all of one type."""
+    weight (scale_input) or the product times it.  h [T, d]; w_up [E, F, d]; w_down [E, d, F], all of one type.
+    gated: w_up is [E, 2 F, d], an expert's gate rows then its up rows, and the activation joins the two."""
     T, d = h.shape
     E, F, _ = w_up.shape
+    if gated:
+        if F % 2:
+            raise KernelError("moe_experts: a gated expert's first matrix holds gate and up rows, an even number")
+        F //= 2
     top = ids.shape[1]
     dt = h.dtype
     _gpu("h", h)
-    _gpu("w_up", w_up, dt, (E, F, d))
+    _gpu("w_up", w_up, dt, (E, 2 * F if gated else F, d))
     _gpu("w_down", w_down, dt, (E, d, F))
     _gpu("ids", ids, torch.int32, (T, top))
     _gpu("wts", wts, torch.float32, (T, top))
@@ -1246,7 +1395,8 @@ def moe_experts(h, w_up, w_down, ids, wts, residual, *, activation: str = "relu2
     y = torch.empty(T * top, d, dtype=torch.float32, device=h.device)
     _check(load("moe").tuff_moe_experts(h.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), _dt(h), ids.data_ptr(),
                                         wts.data_ptr(), a.data_ptr(), y.data_ptr(), residual.data_ptr(), T, d, F, top,
-                                        {"relu2": 0, "silu": 1, "gelu_tanh": 2}[activation], int(scale_input), _stream()),
+                                        _expert_activation(activation, gated, limit), int(scale_input), int(gated),
+                                        float(limit), float(alpha), _stream()),
            "moe_experts")
 
 

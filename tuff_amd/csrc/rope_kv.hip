@@ -46,14 +46,14 @@ __global__ __launch_bounds__(POST_WAVES * WAVE) void qkv_post_kernel(
     const float* __restrict__ inv_freq, int rotary_dim, int interleaved,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping,
     int H, int Hkv, int hd, int page_size, int heads, int heads_per_wave,
-    const float* __restrict__ angles, int n_angles) {
+    const float* __restrict__ angles, int n_angles, int row_stride) {
     __shared__ float vals_all[POST_WAVES][MAX_PER_LANE * WAVE];
     const int t = blockIdx.x, lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
     float* vals = vals_all[wave];
     const int head_begin = (blockIdx.y * POST_WAVES + wave) * heads_per_wave;
     const int head_end = min(heads, head_begin + heads_per_wave);
     if (head_begin >= head_end) return;
-    const int row_width = (H + 2 * Hkv) * hd;
+    const int row_width = row_stride > 0 ? row_stride : (H + 2 * Hkv) * hd;      // (a row may hold more behind its q and k heads)
     const int half = rotary_dim / 2;
 
     // rotation of element j = lane + 64 i: which frequency, which partner, cosine and sine
@@ -321,11 +321,14 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
                               const float* inv_freq, int rotary_dim, int interleaved,
                               const int* positions, const int* slot_mapping,
                               int n_tokens, int H, int Hkv, int hd, int page_size,
-                              const float* angles, int n_angles, hipStream_t stream) {
+                              const float* angles, int n_angles, int row_stride, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (hd > MAX_PER_LANE * WAVE || rotary_dim > hd || (rotary_dim % 2) != 0) return -2;
+    // row_stride > 0: elements from a token's row to the next, where that is not (H + 2 Hkv) hd (values of another
+    // width behind the keys: then nothing is written to the cache here, only q_out and k_out)
+    if (row_stride > 0 && (k_cache || row_stride < (H + Hkv) * hd)) return -2;
     if (!angles || !inv_freq) n_angles = 0;              // [n_angles][2][rotary_dim / 2] as tuff_rope_table makes it
-    if (hd == 64 && inv_freq && rotary_dim == 64 && !interleaved && !k_out && page_size % 16 == 0) {
+    if (hd == 64 && inv_freq && rotary_dim == 64 && !interleaved && !k_out && page_size % 16 == 0 && row_stride <= 0) {
         // shares of a token's heads: enough sixteen-lane groups for the chip, whole heads each
         const int n_heads = k_cache ? H + Hkv : H;
         int shares = 1;
@@ -351,7 +354,7 @@ TUFF_EXPORT int tuff_qkv_post(const void* qkv, void* q_out, void* k_out, void* k
     dim3 grid(n_tokens, ceil_div(heads, POST_WAVES * heads_per_wave)), block(POST_WAVES * WAVE);
 #define LAUNCH(T, TW) hipLaunchKernelGGL((qkv_post_kernel<T, TW>), grid, block, 0, stream, (const T*)qkv, (T*)q_out, (T*)k_out, \
         (T*)k_cache, (T*)v_cache, (const TW*)q_norm_w, (const TW*)k_norm_w, eps, inv_freq, rotary_dim, interleaved, \
-        positions, slot_mapping, H, Hkv, hd, page_size, heads, heads_per_wave, angles, n_angles)
+        positions, slot_mapping, H, Hkv, hd, page_size, heads, heads_per_wave, angles, n_angles, row_stride)
     if (dt == DT_F32 && norm_dt == DT_F32) LAUNCH(float, float);
     else if (dt == DT_F32) LAUNCH(float, bf16_t);
     else if (norm_dt == DT_F32) LAUNCH(bf16_t, float);

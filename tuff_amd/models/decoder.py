@@ -33,15 +33,26 @@ class DecoderModel:
                  blocks: list[Block], final_norm: Norm, head: Optional[WeightDecl] = None,
                  schedule: Optional[list[LayerRun]] = None, max_positions: Optional[int] = None,
                  eos_token_id: Optional[int] = None, embedding_scale: float = 1.0,
-                 logit_scale: float = 1.0, logit_softcap: Optional[float] = None, pad_hidden: bool = False):
+                 logit_scale: float = 1.0, logit_softcap: Optional[float] = None, pad_hidden: bool = False,
+                 streams: Optional[int] = None):
         """head=None: the head is the embedding (tied), as the reference does when the file has
         no output matrix (src/lfm25_model.c:128-131).
         embedding_scale: the embedding rows are multiplied by it on their way into the residual stream.
         logit_scale, logit_softcap: logits = head(norm(x)) * logit_scale, then, with a cap c,
         c * tanh(logits / c).  The reference has none of the three (scale 1, no cap), which are the defaults.
         pad_hidden: a hidden size that is no multiple of 8 is served in bfloat16 too, by zero columns (for a
-        model all of whose parts take such a size); without it such a model is refused when it is bound."""
+        model all of whose parts take such a size); without it such a model is refused when it is bound.
+        streams: the model keeps that many residual streams [S, T, d], all equal to the embedding at the start
+        and summed before the final norm; its blocks are then all of a kind that takes them (multi_stream)."""
         self.pad_hidden = bool(pad_hidden)
+        self.streams = None if streams is None else int(streams)
+        if self.streams is not None and (self.streams < 1 or not all(getattr(b, "multi_stream", False) for b in blocks)):
+            raise ValueError("a model with several residual streams needs at least one and blocks that take them")
+        if self.streams is None and any(getattr(b, "multi_stream", False) for b in blocks):
+            raise ValueError("a block over several residual streams in a model that keeps one")
+        #: debugging aid: called as on_layer(run index, x [T, d] or xs [S, T, d]) after every layer run; while it
+        #: is set no step is recorded into a graph
+        self.on_layer = None
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.embedding_decl, self.head_decl = embedding, head
         self.blocks, self.final_norm = list(blocks), final_norm
@@ -117,7 +128,7 @@ class DecoderModel:
         return merge_token_inputs([t for b in self.blocks for t in b.token_inputs()])
 
     def graph_safe(self) -> bool:
-        return all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe
+        return self.on_layer is None and all(b.graph_safe for b in self.blocks) and self.final_norm.graph_safe
 
     def records_portions(self) -> bool:
         return self.graph_safe() and all(getattr(b, "records_portions", False) for b in self.blocks)
@@ -140,6 +151,8 @@ class DecoderModel:
             b.bind(weights, rt)
         self.final_norm.bind(weights, rt)
         self._head_cast: Optional[torch.Tensor] = None
+        if self.streams is not None:
+            self._ones = torch.ones(self.streams, dtype=torch.float32, device=rt.device)
         if self.head.dtype != rt.dtype and self.head.dtype != torch.float32:
             raise TypeError(f"head weight of type {self.head.dtype} in a {rt.dtype} run")
         self._head_k = self.hidden_size
@@ -162,6 +175,9 @@ class DecoderModel:
         """Runs the step's tokens through all layers.  Returns float32 logits
         [len(ctx.logit_rows), vocab], or None when no logits are wanted."""
         rt = self.rt
+        if self.streams is not None:
+            x = self._forward_streams(ctx, cache_views)
+            return self._finish(x, ctx, False, False)
         x = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=rt.device)
         ops.embed_rows(self.embedding, ctx.tokens, x, self.embedding_scale)
         head_fused, all_rows = self._head_fused(ctx)
@@ -176,6 +192,32 @@ class DecoderModel:
                 block.forward(x, ctx, self._views_of(i, cache_views), run.writes, next_norm=nxt)
             else:
                 block.forward(x, ctx, self._views_of(i, cache_views), run.writes)
+            if self.on_layer is not None:
+                self.on_layer(i, x)
+        return self._finish(x, ctx, head_fused, all_rows)
+
+    def _forward_streams(self, ctx, cache_views) -> torch.Tensor:
+        """The layers over several residual streams; returns the sum of the streams, float32 [T, d].  The kernel that
+        writes a block's last output into the streams also reads the next block's first input (or the final sum)."""
+        S = self.streams
+        xs = torch.empty(S, ctx.T, self.hidden_size, dtype=torch.float32, device=self.rt.device)
+        for s in range(S):
+            ops.embed_rows(self.embedding, ctx.tokens, xs[s], self.embedding_scale)
+        carry = None
+        last = len(self.schedule) - 1
+        for i, run in enumerate(self.schedule):
+            block = self.blocks[run.block]
+            nxt = self.blocks[self.schedule[i + 1].block].first_read() if i < last else (self._ones, None, 0.0)
+            carry = block.forward(xs, ctx, self._views_of(i, cache_views), run.writes, carry=carry, next_read=nxt)
+            if self.on_layer is not None:
+                self.on_layer(i, xs)
+        if last < 0:
+            carry = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=self.rt.device)
+            ops.hc_step(xs, in_w=self._ones, u_out=carry)
+        return carry
+
+    def _finish(self, x, ctx, head_fused: bool, all_rows: bool) -> Optional[torch.Tensor]:
+        """The final norm and the head over x float32 [T, d]."""
         # which rows are wanted is a fact of the step, not of its shape: the head runs outside of what is recorded
         # (a recorder keeps the function and hands back what it returns at each replay)
         # What the last block left for the final norm is taken here, where the step's kernels are issued (or

@@ -71,6 +71,9 @@ def _register_builtin() -> None:
     from ..config.pafodra import PafodraConfig
     from .pafodra import build_pafodra
     register_architecture(PafodraConfig.architecture, PafodraConfig, build_pafodra)
+    from ..config.kugalorn import KugalornConfig
+    from .kugalorn import build_kugalorn
+    register_architecture(KugalornConfig.architecture, KugalornConfig, build_kugalorn)
 
 
 _register_builtin()

@@ -4,7 +4,9 @@ q = W_q h, k = W_k h, v = W_v h; optional per-head RMSNorm of q and k with a sha
 weight; optional position encoding; k (normed, encoded) and v (as projected) go to the cache
 at the token's slot; every token attends to the cached keys of its request up to its own
 position (within `window` if given); query head i reads kv head i // (H / Hkv); scores are
-scaled by 1/sqrt(hd); o = W_o concat(heads).
+scaled by 1/sqrt(hd); o = W_o concat(heads).  Options: a per-head norm of q and k without a
+weight (unit root mean square), and a distance penalty slope_h * (i - j) taken off the scaled
+score of query i and key j, slope_h = 2^(-span (h + 1) / H).
 Reference: src/lfm25_engine.c:386-405, src/lfm25_gpu.cu:420-485, :506-558.
 """
 from __future__ import annotations
@@ -29,9 +31,11 @@ class AttentionMixer(Mixer):
                  names: dict[str, str], qk_norm_eps: Optional[float] = None,
                  position: Optional[PositionEncoding] = None, window: Optional[int] = None,
                  scale: Optional[float] = None, aliases: Optional[dict[str, tuple]] = None,
-                 value_dim: Optional[int] = None):
-        """names: checkpoint names of 'q', 'k', 'v', 'o' and, with qk_norm_eps, 'q_norm', 'k_norm'; with a
-        'sink' among them the heads have sinks.  value_dim: width of a value head (default: head_dim)."""
+                 value_dim: Optional[int] = None, slope_span: Optional[float] = None):
+        """names: checkpoint names of 'q', 'k', 'v', 'o' and, with qk_norm_eps, 'q_norm', 'k_norm' (without these
+        two names the norm has no weight: q and k are divided by their root mean square over the head); with a
+        'sink' among them the heads have sinks.  value_dim: width of a value head (default: head_dim).
+        slope_span: heads have distance slopes 2^(-slope_span (h + 1) / H) (None: none)."""
         if num_heads % num_kv_heads:
             raise ValueError(f"heads {num_heads} must be a multiple of kv heads {num_kv_heads}")
         if head_dim > 256:
@@ -40,10 +44,12 @@ class AttentionMixer(Mixer):
         self.vd = self.hd if value_dim is None else int(value_dim)
         if self.vd > 256 or self.vd < 1:
             raise ValueError(f"value size {self.vd} is outside 1..256")
-        if self.vd != self.hd and (qk_norm_eps is not None or position is not None):
-            raise ValueError("values of another width than keys go with plain queries and keys only (no per-head "
-                             "norm, no position encoding)")
+        if self.vd != self.hd and position is not None:
+            raise ValueError("values of another width than keys go with no position encoding")
         self.has_sink = "sink" in names
+        self.norm_has_weight = qk_norm_eps is not None and "q_norm" in names
+        self.slope_span = None if slope_span is None else float(slope_span)
+        self.slopes = None
         self.sinks = None
         self.eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.position, self.window = position, (int(window) if window else None)
@@ -67,7 +73,7 @@ class AttentionMixer(Mixer):
 
     def weight_decls(self):
         decls = self.qkv.weight_decls() + self.out.weight_decls()
-        if self.eps is not None:
+        if self.norm_has_weight:
             decls += [WeightDecl(self.names["q_norm"], (self.hd,), "norm", aliases=self._al.get("q_norm", ())),
                       WeightDecl(self.names["k_norm"], (self.hd,), "norm", aliases=self._al.get("k_norm", ()))]
         if self.position is not None:
@@ -77,7 +83,9 @@ class AttentionMixer(Mixer):
         return decls
 
     def kernel_modules(self):
-        mods = ["rope_kv", "attention", "attention_mfma", "attention_prefill"]
+        mods = ["rope_kv", "attention"]
+        if self.slope_span is None:
+            mods += ["attention_mfma", "attention_prefill"]       # (the matrix-core kernels know no distance slopes)
         if self.position is not None:
             mods += self.position.kernel_modules()
         return mods
@@ -92,12 +100,18 @@ class AttentionMixer(Mixer):
         self.rt = rt
         self.qkv.bind(weights, rt)
         self.out.bind(weights, rt)
-        if self.eps is not None:
+        if self.norm_has_weight:
             self.q_norm_w = weights[self.names["q_norm"]]
             self.k_norm_w = weights[self.names["k_norm"]]
             if self.q_norm_w.dtype != self.k_norm_w.dtype:
                 self.q_norm_w = self.q_norm_w.float()
                 self.k_norm_w = self.k_norm_w.float()
+        elif self.eps is not None:
+            self.q_norm_w = self.k_norm_w = torch.ones(self.hd, dtype=torch.float32, device=rt.device)
+        if self.slope_span is not None:
+            # in float64, then rounded once
+            self.slopes = torch.tensor([2.0 ** (-self.slope_span * (h + 1) / self.H) for h in range(self.H)],
+                                       dtype=torch.float64).to(torch.float32).to(rt.device)
         if self.position is not None:
             self.position.bind(weights, rt)
         if self.has_sink:
@@ -122,10 +136,14 @@ class AttentionMixer(Mixer):
             """What depends on where the step's tokens lie: positions, cache slots, block tables."""
             g = ctx.groups[cache.group]
             if vd != hd:
-                # keys and values of different widths: the rows are cut out and written as they are
-                qq = qkv[:, :H * hd].contiguous()
+                # keys and values of different widths: the rows are cut out (normed, where there is a norm) and written
+                if self.eps is not None:
+                    qq, kk = self.rt.empty(T, H * hd), self.rt.empty(T, Hkv * hd)
+                    ops.qkv_post(qkv, qq, H=H, Hkv=Hkv, hd=hd, positions=ctx.positions, k_out=kk, wide_rows=True, **norm)
+                else:
+                    qq, kk = qkv[:, :H * hd].contiguous(), qkv[:, H * hd:(H + Hkv) * hd].contiguous()
                 if write_cache:
-                    ops.kv_write(qkv[:, H * hd:(H + Hkv) * hd].contiguous(), qkv[:, (H + Hkv) * hd:].contiguous(),
+                    ops.kv_write(kk, qkv[:, (H + Hkv) * hd:].contiguous(),
                                  cache.k, cache.v, g.slot_mapping, Hkv=Hkv, hd=hd, vd=vd, page_size=cache.page_size)
                 self.attend(qq, o, ctx, cache, g)
                 return
@@ -200,7 +218,7 @@ class AttentionMixer(Mixer):
 
     def attend(self, q, o, ctx, cache, g) -> None:
         G = self.H // self.Hkv
-        if self.vd == self.hd and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
+        if self.vd == self.hd and self.slopes is None and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
             common = dict(block_table=g.block_table, req_info=ctx.req_info, H=self.H, Hkv=self.Hkv, hd=self.hd,
                           page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
                           scale=self.scale, sinks=self.sinks)
@@ -226,4 +244,4 @@ class AttentionMixer(Mixer):
         ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
                               req_of_token=ctx.req_of_token, positions=ctx.positions,
                               H=self.H, Hkv=self.Hkv, hd=self.hd, page_size=cache.page_size,
-                              window=self.window or 0, scale=self.scale, vd=self.vd, sinks=self.sinks)
+                              window=self.window or 0, scale=self.scale, vd=self.vd, sinks=self.sinks, slopes=self.slopes)

@@ -20,7 +20,7 @@ class WeightDecl:
     """One tensor a part needs from the checkpoint."""
     name: str                       # name in the checkpoint
     shape: tuple
-    init: str = "normal"            # random-weights mode: "normal" N(0, 0.02) | "norm" 1 + N(0, 0.01)
+    init: str = "normal"            # random-weights mode: "normal" N(0, 0.02) | "norm" 1 + N(0, 0.01) | "around:<m>" m + N(0, 0.01) | "identity"
     alt_shapes: tuple = ()          # shapes that are accepted and reshaped to `shape`
     aliases: tuple = ()             # other names the same tensor may have
     role: str = ""                  # "projection": the matrix of a Linear (every token is multiplied by it)
@@ -34,16 +34,24 @@ class PagedKV:
     ([page, kv_head, offset, value_dim]), instead of transposed within the page ([page, kv_head,
     value_dim, offset], which is what the matrix cores of the framework's own attention kernels
     read).  Those kernels take equal widths and transposed values only and refuse another cache by
-    its shape; a mixer with kernels of its own declares what suits them."""
+    its shape; a mixer with kernels of its own declares what suits them.  `values_in_keys`: nothing is kept
+    beside the key rows (a latent row a position that is key and value at once: the values are its first
+    value_dim channels); the view's `v` is then None."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None
     value_rows: bool = False
+    values_in_keys: bool = False
 
     @property
     def v_dim(self) -> int:
         return self.head_dim if self.value_dim is None else self.value_dim
+
+    @property
+    def elements_per_token(self) -> int:
+        """Cache elements one token costs in this entry."""
+        return self.num_kv_heads * (self.head_dim + (0 if self.values_in_keys else self.v_dim))
 
 
 @dataclasses.dataclass(frozen=True)

@@ -6,12 +6,19 @@ with the residual stream x in float32.  A feed-forward of None leaves out the se
 
 ParallelBlock has one norm whose output both sublayers read:
     h = norm(x);  x += mixer(h) + ffn(h)
+
+HyperConnectionBlock is the pre-norm layer over several residual streams: a sublayer reads a weighted sum
+of the streams and its output goes back into all of them through a mixing matrix.
 """
 from __future__ import annotations
 
 from typing import Optional
 
-from .base import BLOCKS, Block, FeedForward, Mixer, Norm, Runtime
+import torch
+
+from ..csrc import ops
+from .base import BLOCKS, Block, FeedForward, Mixer, Norm, Runtime, WeightDecl
+from .norm import RMSNorm
 
 
 @BLOCKS.register("prenorm")
@@ -129,3 +136,107 @@ class ParallelBlock(Block):
         if self.ffn is not None:
             kw = {"next_norm": None} if self.ffn.adds_once_through_linear else {}
             self.ffn.forward(h, ctx, x, **kw)
+
+
+@BLOCKS.register("hyper")
+class HyperConnectionBlock(Block):
+    """A pre-norm layer over S residual streams xs [S, T, d] instead of one.  For sublayer q (1: the mixer, 2: the
+    feed-forward) with its three tensors in_q [S], mix_q [S, S] (indexed [from, to]) and out_q [S]:
+        u = sum_s in_q[s] xs[s];   y = sublayer(norm_q(u));   xs[r] <- sum_s mix_q[s, r] xs[s] + out_q[r] y
+    (all streams at once, from the old values).  ffn None: the mixer's sublayer alone.
+
+    One kernel writes a sublayer's output into the streams and reads the next sublayer's input with its norm
+    (ops.hc_step); the next sublayer may be the next block's first, so forward() takes what the block before left
+    (`carry`) and is told who reads next (`next_read`).  names: checkpoint names 'in1', 'mix1', 'out1' and, with
+    a feed-forward, 'in2', 'mix2', 'out2'."""
+    multi_stream = True
+
+    def __init__(self, streams: int, norm1: Norm, mixer: Mixer, norm2: Optional[Norm] = None,
+                 ffn: Optional[FeedForward] = None, *, names: dict[str, str]):
+        if (norm2 is None) != (ffn is None):
+            raise ValueError("norm2 and ffn go together")
+        self.S = int(streams)
+        if self.S < 1:
+            raise ValueError("at least one stream")
+        for n in (norm1, norm2):
+            if n is not None and not isinstance(n, RMSNorm):
+                raise ValueError("the norms of a hyper-connection block are RMS norms (they run inside the streams' kernel)")
+        self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
+        self.names = dict(names)
+
+    def _parts(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.ffn) if p is not None]
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self._parts())
+
+    @property
+    def records_portions(self):
+        return all(p.records_portions for p in self._parts())
+
+    def weight_decls(self):
+        S = self.S
+        decls = [d for p in self._parts() for d in p.weight_decls()]
+        for q in ("1", "2") if self.ffn is not None else ("1",):
+            decls += [WeightDecl(self.names["in" + q], (S,), f"around:{1.0 / S}"),
+                      WeightDecl(self.names["out" + q], (S,), "norm"),
+                      WeightDecl(self.names["mix" + q], (S, S), "identity")]
+        return decls
+
+    def kernel_modules(self):
+        return ["hyper", "elementwise"] + [m for p in self._parts() for m in p.kernel_modules()]
+
+    def token_inputs(self):
+        return [t for p in self._parts() for t in p.token_inputs()]
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        for p in self._parts():
+            p.bind(weights, rt)
+        f32 = lambda name: weights[self.names[name]].to(torch.float32).contiguous()
+        self.hc = {q: (f32("in" + q), f32("mix" + q), f32("out" + q)) for q in (("1", "2") if self.ffn is not None else ("1",))}
+
+    def first_read(self):
+        """(in [S], norm weight float32 [d], eps): what the block before needs to prepare this block's first input."""
+        return self.hc["1"][0], self.norm1.weight_f32, self.norm1.eps
+
+    def forward(self, xs, ctx, cache, write_cache: bool = True, carry=None, next_read=None):
+        """xs float32 [S, T, d], in place.  carry: norm1(u) of this block's first sublayer where the block before
+        left it (None: computed here).  next_read: (in, norm weight or None, eps) of whoever reads the streams
+        next; the result of that read is returned (the normed rows in the compute type, or, without a norm weight,
+        the plain weighted sum in float32); None: nothing is read."""
+        S, T, d = xs.shape
+        if S != self.S:
+            raise ValueError(f"{S} streams handed to a block of {self.S}")
+        if carry is None:
+            carry = self.rt.empty(T, d)
+            in1, w1, eps1 = self.first_read()
+            ops.hc_step(xs, in_w=in1, norm_w=w1, eps=eps1, h_out=carry)
+        y = torch.empty(T, d, dtype=torch.float32, device=xs.device)
+        ops.fill_u32(y, 0)
+        kw = {"next_norm": None} if self.mixer.adds_once_through_linear else {}
+        self.mixer.forward(carry, ctx, cache, y, write_cache, **kw)
+        _, mix1, out1 = self.hc["1"]
+        if self.ffn is None:
+            return self._write_and_read(xs, y, mix1, out1, next_read)
+        in2, mix2, out2 = self.hc["2"]
+        h = self._write_and_read(xs, y, mix1, out1, (in2, self.norm2.weight_f32, self.norm2.eps))
+        ops.fill_u32(y, 0)
+        kw = {"next_norm": None} if self.ffn.adds_once_through_linear else {}
+        self.ffn.forward(h, ctx, y, **kw)
+        return self._write_and_read(xs, y, mix2, out2, next_read)
+
+    def _write_and_read(self, xs, y, mix, out_w, read):
+        T, d = y.shape
+        if read is None:
+            ops.hc_step(xs, y=y, mix=mix, out_w=out_w)
+            return None
+        in_w, norm_w, eps = read
+        if norm_w is None:
+            u = torch.empty(T, d, dtype=torch.float32, device=xs.device)
+            ops.hc_step(xs, y=y, mix=mix, out_w=out_w, in_w=in_w, u_out=u)
+            return u
+        h = self.rt.empty(T, d)
+        ops.hc_step(xs, y=y, mix=mix, out_w=out_w, in_w=in_w, norm_w=norm_w, eps=eps, h_out=h)
+        return h

@@ -75,17 +75,21 @@ class SwiGLU(FeedForward):
 @FEED_FORWARDS.register("gated")
 class GatedMLP(FeedForward):
     """W_down (act(W_gate h + b_gate) * (W_up h + b_up)) + b_down.  activation: "silu" or "gelu_tanh"
-    (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))).  names: 'gate', 'up' [F, d], 'down' [d, F] and, with
-    bias=True, 'gate.b', 'up.b' [F], 'down.b' [d]."""
+    (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))), or "swish_clamp": with g = min(W_gate h, limit) and
+    u = clamp(W_up h, -limit, limit) the product is g sigmoid(alpha g) (u + 1).  names: 'gate', 'up' [F, d],
+    'down' [d, F] and, with bias=True, 'gate.b', 'up.b' [F], 'down.b' [d]."""
     graph_safe = True
     records_portions = True
     adds_once_through_linear = True
 
     def __init__(self, hidden_size: int, ffn_dim: int, *, names: dict[str, str], activation: str = "gelu_tanh",
-                 bias: bool = False):
-        if activation not in ("silu", "gelu_tanh"):
+                 bias: bool = False, limit: float = 0.0, alpha: float = 1.0):
+        if activation not in ("silu", "gelu_tanh", "swish_clamp"):
             raise ValueError(f"unknown activation '{activation}'")
+        if activation == "swish_clamp" and not limit > 0:
+            raise ValueError("the clamped activation needs a positive limit")
         self.d, self.F, self.activation, self.has_bias = int(hidden_size), int(ffn_dim), activation, bool(bias)
+        self.limit, self.alpha = float(limit), float(alpha)
         self._names = dict(names)
         self._make(self.F)
         self._decls = self.gate_up.weight_decls() + self.down.weight_decls()
@@ -128,7 +132,7 @@ class GatedMLP(FeedForward):
     def forward(self, h, ctx, residual, next_norm=None) -> None:
         gu = self.gate_up.forward(h, out_dtype=torch.float32)       # the activation reads the sums as they are, plus the biases
         act = self.rt.empty(h.shape[0], self.width)
-        ops.glu(gu, act, self.activation, self.gu_bias)
+        ops.glu(gu, act, self.activation, self.gu_bias, limit=self.limit, alpha=self.alpha)
         self.down.forward(act, accumulate_into=residual, next_norm=next_norm)
 
 
@@ -142,22 +146,34 @@ class MoE(FeedForward):
     else its output.  The shared expert runs for every token and is multiplied by sigmoid(W_sg h), one number a
     token (names['shared.sg'], [1, d]); without that name it is added as it is.
     names: 'router' [E, d]; 'experts': a list of (up [F, d], down [d, F]) names; optional 'shared.up',
-    'shared.down', 'shared.sg'."""
+    'shared.down', 'shared.sg'; optional 'router.b' [E], a bias on the router's logits.
+    gated: an expert is W_down glu(W_gate x, W_up x) and 'experts' lists (gate, up, down) names; glu(g, u) is
+    act(g) u, or, activation "swish_clamp", g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit) and
+    u' = clamp(u, -limit, limit).  shared: a feed-forward of any kind that runs for every token and is added (in
+    place of the built-in ungated one that shared_dim asks for)."""
     graph_safe = True
     records_portions = True
 
     def __init__(self, hidden_size: int, num_experts: int, top: int, expert_dim: int, *, names: dict,
                  activation: str = "relu2", router_weights: str = "sigmoid", scale_input: bool = True,
-                 shared_dim: int = 0):
+                 shared_dim: int = 0, gated: bool = False, limit: float = 0.0, alpha: float = 1.0,
+                 shared: FeedForward | None = None):
         self.d, self.E, self.top, self.F = int(hidden_size), int(num_experts), int(top), int(expert_dim)
         if not 1 <= self.top <= self.E:
             raise ValueError(f"top {self.top} of {self.E} experts")
-        if activation not in ("relu2", "silu", "gelu_tanh"):
+        if activation not in ("relu2", "silu", "gelu_tanh", "swish_clamp"):
             raise ValueError(f"unknown activation '{activation}'")
+        self.gated, self.limit, self.alpha = bool(gated), float(limit), float(alpha)
+        if activation == "swish_clamp" and (not self.gated or not self.limit > 0):
+            raise ValueError("the clamped activation is for gated experts and needs a positive limit")
         self.activation, self.router_weights, self.scale_input = activation, router_weights, bool(scale_input)
         self.names = dict(names)
-        if len(self.names["experts"]) != self.E:
-            raise ValueError("one (up, down) pair of names per expert")
+        if len(self.names["experts"]) != self.E or any(len(e) != (3 if self.gated else 2) for e in self.names["experts"]):
+            raise ValueError("one (up, down) pair of names per expert ((gate, up, down) for gated experts)")
+        if shared is not None and shared_dim:
+            raise ValueError("either a shared feed-forward of its own or shared_dim")
+        self.shared = shared
+        self.has_router_bias = "router.b" in self.names
         self.Fs = int(shared_dim)
         self.shared_gate = self.Fs > 0 and "shared.sg" in self.names
         self.shared_up = self.shared_down = None
@@ -172,31 +188,43 @@ class MoE(FeedForward):
         decls = [WeightDecl(self.names["router"], (self.E, self.d), "normal", role="projection")]
         if self.shared_gate:
             decls.append(WeightDecl(self.names["shared.sg"], (1, self.d), "normal", role="projection"))
-        for up, down in self.names["experts"]:
-            decls += [WeightDecl(up, (self.F, self.d), "normal", role="projection"),
-                      WeightDecl(down, (self.d, self.F), "normal", role="projection")]
+        if self.has_router_bias:
+            decls.append(WeightDecl(self.names["router.b"], (self.E,), "normal"))
+        for e in self.names["experts"]:
+            decls += [WeightDecl(n, (self.F, self.d), "normal", role="projection") for n in e[:-1]]
+            decls.append(WeightDecl(e[-1], (self.d, self.F), "normal", role="projection"))
+        if self.shared is not None:
+            decls += self.shared.weight_decls()
         if self.Fs:
             decls += [WeightDecl(self.names["shared.up"], (self.Fs, self.d), "normal", role="projection"),
                       WeightDecl(self.names["shared.down"], (self.d, self.Fs), "normal", role="projection")]
         return decls
 
     def kernel_modules(self):
-        return ["moe", "elementwise"]
+        return ["moe", "elementwise"] + (self.shared.kernel_modules() if self.shared is not None else [])
 
     def bind(self, weights, rt: Runtime):
         self.rt = rt
         # the router's rows (and the shared expert's gate row behind them) stay float32: their products decide
         rows = [weights[self.names["router"]]] + ([weights[self.names["shared.sg"]]] if self.shared_gate else [])
         self.router_w = torch.cat([r.to(torch.float32).reshape(-1, self.d) for r in rows]).contiguous()
-        ups = [weights[up] for up, _ in self.names["experts"]]
-        downs = [weights[down] for _, down in self.names["experts"]]
+        self.router_b = weights[self.names["router.b"]].to(torch.float32).contiguous() if self.has_router_bias else None
+        ups = [weights[e[-2]] for e in self.names["experts"]]
+        gates = [weights[e[0]] for e in self.names["experts"]] if self.gated else None
+        downs = [weights[e[-1]] for e in self.names["experts"]]
         self.grouped = ops.moe_grouped_supported(ups[0].dtype, self.d, self.F, self.E) and rt.dtype == torch.bfloat16
         if self.grouped:
-            # the matrix cores' order, an expert after the other
+            # the matrix cores' order, an expert after the other; a gated expert's gate and up rows take turns
+            if self.gated:
+                ups = [ops.interleave_gate_up(g, u) for g, u in zip(gates, ups)]
             self.up_tiles, self.down_tiles = ops.tile_experts(ups), ops.tile_experts(downs)
         else:
-            self.w_up = torch.stack(ups).contiguous()                # [E, F, d]
+            if self.gated:
+                ups = [torch.cat([g, u]) for g, u in zip(gates, ups)]        # an expert's gate rows, then its up rows
+            self.w_up = torch.stack(ups).contiguous()                # [E, F or 2 F, d]
             self.w_down = torch.stack(downs).contiguous()            # [E, d, F]
+        if self.shared is not None:
+            self.shared.bind(weights, rt)
         if self.Fs:
             up, down = weights[self.names["shared.up"]], weights[self.names["shared.down"]]
             if self.Fs % 8 and up.dtype == torch.bfloat16 and down.dtype == torch.bfloat16:
@@ -213,13 +241,15 @@ class MoE(FeedForward):
         z = torch.empty(T, self.router_w.shape[0], dtype=torch.float32, device=h.device)        # [T, E (+ 1)]
         ids = torch.empty(T, self.top, dtype=torch.int32, device=h.device)
         wts = torch.empty(T, self.top, dtype=torch.float32, device=h.device)
-        ops.moe_router(h, self.router_w, z, ids, wts, E=self.E, top=self.top, weights=self.router_weights)
+        ops.moe_router(h, self.router_w, z, ids, wts, E=self.E, top=self.top, weights=self.router_weights, bias=self.router_b)
+        form = dict(activation=self.activation, scale_input=self.scale_input, gated=self.gated, limit=self.limit, alpha=self.alpha)
         if self.grouped:
-            ops.moe_experts_grouped(h, self.up_tiles, self.down_tiles, ids, wts, residual, F=self.F,
-                                    activation=self.activation, scale_input=self.scale_input)
+            ops.moe_experts_grouped(h, self.up_tiles, self.down_tiles, ids, wts, residual, F=self.F, **form)
         else:
-            ops.moe_experts(h, self.w_up, self.w_down, ids, wts, residual, activation=self.activation,
-                            scale_input=self.scale_input)
+            ops.moe_experts(h, self.w_up, self.w_down, ids, wts, residual, **form)
+        if self.shared is not None:
+            kw = {"next_norm": None} if self.shared.adds_once_through_linear else {}
+            self.shared.forward(h, ctx, residual, **kw)
         if self.Fs:
             a = self.shared_up.forward(h)
             # the gate is one number a token and the second product is linear: it goes onto the activations

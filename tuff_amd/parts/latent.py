@@ -1,0 +1,111 @@
+"""Latent attention mixer over the paged cache.
+
+Keys and values are expansions of one narrow row a token: with h the mixer's input,
+    [c_raw | k_r] = W_dkv h,   c = rmsnorm(c_raw) * w   (rank channels),   k_r rotated (rot channels, shared by all heads)
+    head a:  key = [W_uk,a c | k_r],  value = W_uv,a c,  query = [q_plain,a | rotate(q_rot,a)] from W_q h
+    score = (query . key) * scale, causal softmax, head output times sigmoid((W_g h)_a) (where there is a gate), W_o.
+The cache keeps [c | k_r] and nothing else: rank + rot numbers a token, one "kv head" for all query
+heads, the row's first `rank` channels serving as the value.  The expansions are never formed for the
+cached tokens: the query is carried into the latent space, q' = [W_uk,a^T q_plain,a | q_rot,a], attention
+runs over the cache rows as they lie, and W_uv,a is applied to the head's weighted sum of rows.
+
+Rotation: neighbouring pairs (2i, 2i + 1) of the first `rot_dims` channels of the rotated part turn by
+position * base^(-2i / rot_dims); the rest passes.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..csrc import ops
+from .base import MIXERS, Mixer, PagedKV, Runtime, WeightDecl
+from .linear import Linear
+
+
+@MIXERS.register("latent_attention")
+class LatentAttentionMixer(Mixer):
+    graph_safe = True
+    records_portions = True
+    accepts_pending_norm = True
+    adds_once_through_linear = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, value_dim: int, rank: int, *,
+                 names: dict[str, str], norm_eps: float, scale: float, rot_base: float, rot_dims: Optional[int] = None,
+                 window: Optional[int] = None):
+        """names: checkpoint names of 'q' [H (dim + rot), d], 'dkv' [rank + rot, d], 'dkv.norm' [rank],
+        'uk' [H dim, rank], 'uv' [H vdim, rank], 'o' [d, H vdim] and, for gated heads, 'g' [H, d].
+        rot_dims: how many of the rot channels turn (default: all)."""
+        self.d, self.H, self.dk, self.dr = int(hidden_size), int(num_heads), int(head_dim), int(rot_dim)
+        self.dv, self.rank = int(value_dim), int(rank)
+        self.lat = self.rank + self.dr
+        self.rot_dims = self.dr if rot_dims is None else int(rot_dims)
+        if self.rot_dims % 2 or not 0 <= self.rot_dims <= self.dr:
+            raise ValueError(f"{self.rot_dims} rotated channels of {self.dr}: an even number within the rotated part is needed")
+        if self.lat > ops.ATTN_GENERAL_MAX_DIM:
+            raise ValueError(f"a latent row of {self.lat} channels is wider than the attention kernels take "
+                             f"({ops.ATTN_GENERAL_MAX_DIM})")
+        if max(self.dk, self.rank) > ops.HEAD_MATMUL_MAX_K:
+            raise ValueError(f"head size {self.dk} / rank {self.rank} above {ops.HEAD_MATMUL_MAX_K}")
+        self.eps, self.scale, self.rot_base = float(norm_eps), float(scale), float(rot_base)
+        self.window = int(window) if window else None
+        self.names = dict(names)
+        self.gated = "g" in self.names
+        ins = [names["q"], names["dkv"]] + ([names["g"]] if self.gated else [])
+        outs = [self.H * (self.dk + self.dr), self.lat] + ([self.H] if self.gated else [])
+        self.proj = Linear(ins, self.d, outs)                       # one product: queries, latent, gates
+        self.out = Linear(names["o"], self.H * self.dv, self.d)
+
+    def weight_decls(self):
+        n = self.names
+        return self.proj.weight_decls() + self.out.weight_decls() + [
+            WeightDecl(n["dkv.norm"], (self.rank,), "norm"),
+            WeightDecl(n["uk"], (self.H * self.dk, self.rank), "normal", role="projection"),
+            WeightDecl(n["uv"], (self.H * self.dv, self.rank), "normal", role="projection")]
+
+    def kernel_modules(self):
+        return ["latent", "attention"]
+
+    def cache_spec(self):
+        return PagedKV(1, self.lat, self.window, value_dim=self.rank, values_in_keys=True)
+
+    def bind(self, weights, rt: Runtime):
+        self.rt = rt
+        self.proj.bind(weights, rt)
+        self.out.bind(weights, rt)
+        n = self.names
+        self.norm_w = weights[n["dkv.norm"]]
+        dt = rt.dtype
+        # W_uk as stored is [H][dim][rank]: k runs over dim, n over rank.  W_uv [H][vdim][rank] is turned per head
+        # to [H][rank][vdim], so that both per-head products read a weight row a step of the inner index.
+        self.w_uk = weights[n["uk"]].to(dt).reshape(self.H, self.dk, self.rank).contiguous()
+        self.w_uv = weights[n["uv"]].to(dt).reshape(self.H, self.dv, self.rank).transpose(1, 2).contiguous()
+        half = self.rot_dims // 2
+        self.inv_freq = torch.tensor([self.rot_base ** (-2.0 * i / self.rot_dims) for i in range(half)],
+                                     dtype=torch.float64).to(torch.float32).to(rt.device)
+
+    def forward(self, h, ctx, cache, residual, write_cache: bool = True, next_norm=None) -> None:
+        T = h.shape[0]
+        H, dk, dr, dv, rank, lat = self.H, self.dk, self.dr, self.dv, self.rank, self.lat
+        proj = self.proj.forward(h)                                           # [T, H (dk + dr) + lat + H]
+        q_width = H * (dk + dr)
+        q_lat = self.rt.empty(T, H * lat)
+        o_lat = self.rt.empty(T, H * rank)
+        o = self.rt.empty(T, H * dv)
+        # the queries' plain parts into the latent space: q'[t, a, :rank] = W_uk,a^T q_plain[t, a]
+        ops.head_matmul(proj, self.w_uk, q_lat, H=H, x_head=dk + dr, y_head=lat)
+
+        def over_the_cache(ctx):
+            g = ctx.groups[cache.group]
+            ops.latent_post(proj, q_lat, cache.k, q_off=0, ckr_off=q_width, norm_w=self.norm_w, eps=self.eps,
+                            inv_freq=self.inv_freq, rot_dims=self.rot_dims, positions=ctx.positions,
+                            slot_mapping=g.slot_mapping if write_cache else None, H=H, dim=dk, rot=dr, rank=rank)
+            ops.attention_general(q_lat, cache.k, None, o_lat, block_table=g.block_table, req_of_token=ctx.req_of_token,
+                                  positions=ctx.positions, H=H, Hkv=1, hd=lat, vd=rank, page_size=cache.page_size,
+                                  window=self.window or 0, scale=self.scale)
+
+        ctx.run_eagerly(over_the_cache)
+        # a head's value expansion of its weighted sum of latent rows, times its gate
+        ops.head_matmul(o_lat, self.w_uv, o, H=H, x_head=rank, y_head=dv,
+                        gate=proj if self.gated else None, gate_col=q_width + lat)
+        self.out.forward(o, accumulate_into=residual, next_norm=next_norm)

@@ -1,6 +1,7 @@
 """Norms of the residual stream, in float32.
 
-RMSNorm: y = x / sqrt(mean(x^2) + eps) * w (src/lfm25_gpu.cu:235,244).
+RMSNorm: y = x / sqrt(mean(x^2) + eps) * w (src/lfm25_gpu.cu:235,244); with offset c the stored weight
+lies around zero and y = x / sqrt(mean(x^2) + eps) * (c + w).
 DynamicTanh: y = tanh(alpha x) w + b with a learned scalar alpha; no mean, no variance.
 """
 from __future__ import annotations
@@ -43,12 +44,14 @@ class RMSNorm(Norm):
     graph_safe = True
     records_portions = True
 
-    def __init__(self, dim: int, eps: float, name: str, aliases: tuple = ()):
+    def __init__(self, dim: int, eps: float, name: str, aliases: tuple = (), offset: float = 0.0):
+        """offset: added to the stored weight (a checkpoint that keeps its norm weights around zero: offset 1)."""
         self.dim, self.eps, self.name, self.aliases = int(dim), float(eps), name, tuple(aliases)
+        self.offset = float(offset)
         self.weight: Optional[torch.Tensor] = None
 
     def weight_decls(self):
-        return [WeightDecl(self.name, (self.dim,), "norm", aliases=self.aliases)]
+        return [WeightDecl(self.name, (self.dim,), "normal" if self.offset else "norm", aliases=self.aliases)]
 
     def kernel_modules(self):
         return ["elementwise"]
@@ -56,6 +59,9 @@ class RMSNorm(Norm):
     def bind(self, weights, rt: Runtime):
         self.rt = rt
         self.weight = weights[self.name]
+        if self.offset:
+            # the sum is float32 whatever the stored type: every kernel that takes this norm reads the sum
+            self.weight = (self.weight.float() + self.offset).contiguous()
         self.weight_f32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float()
 
     def pending(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> PendingNorm:

@@ -1,7 +1,8 @@
 """Random-weights mode: from a configuration and a seed to tensors, or to a model folder
 (config.json + model.safetensors) that loads like any other.
 
-Matrices, embeddings and conv taps are N(0, 0.02); norm weights are 1 + N(0, 0.01).
+Matrices, embeddings and conv taps are N(0, 0.02); norm weights are 1 + N(0, 0.01); a tensor declared
+"around:<m>" is m + N(0, 0.01) and a square one declared "identity" the unit matrix + N(0, 0.01).
 
 The generator is specified down to the bit, so that a seed means the same model wherever and in
 whatever order its tensors are made (host or GPU, whole or in pieces, by this file or by another
@@ -147,7 +148,13 @@ def normal_deviates(key: int, start: int, count: int, device="cpu") -> torch.Ten
 
 
 def random_tensor(decl: WeightDecl, seed: int, dtype: torch.dtype, device="cpu") -> torch.Tensor:
-    if decl.init not in ("norm", "normal"):
+    centre = None
+    if decl.init.startswith("around:"):
+        centre = float(decl.init[len("around:"):])
+    elif decl.init == "identity":
+        if len(decl.shape) != 2 or decl.shape[0] != decl.shape[1]:
+            raise ValueError(f"tensor '{decl.name}': init 'identity' is for square matrices")
+    elif decl.init not in ("norm", "normal"):
         raise ValueError(f"tensor '{decl.name}': unknown init '{decl.init}'")
     shape = tuple(int(n) for n in decl.shape)
     n = math.prod(shape)
@@ -157,7 +164,13 @@ def random_tensor(decl: WeightDecl, seed: int, dtype: torch.dtype, device="cpu")
     for start in range(0, n, chunk):
         count = min(chunk, n - start)
         z = normal_deviates(key, start, count, device)
-        z = 1.0 + STD_NORM * z if decl.init == "norm" else STD_MATRIX * z
+        if centre is not None:
+            z = centre + STD_NORM * z
+        elif decl.init == "identity":
+            at = torch.arange(start, start + count, device=z.device)
+            z = (at // shape[1] == at % shape[1]).to(z.dtype) + STD_NORM * z
+        else:
+            z = 1.0 + STD_NORM * z if decl.init == "norm" else STD_MATRIX * z
         out[start:start + count] = z.to(torch.float32).to(dtype)
     return out.view(shape)
 
