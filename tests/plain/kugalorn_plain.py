@@ -73,7 +73,7 @@ def window_attention(n, W, m, eps, rnd=_same):
     to unit root mean square per head; score = q.k * scale - slope_h * (i - j).  n [T, d]."""
     T = n.shape[0]
     H, G, dk, dv, scale = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"]
-    size = m["mask"]["size"]
+    size = (m.get("mask") or {}).get("size") or T + 1          # no mask: every earlier position
     q = rnd(unit_rms(rnd(n @ W["q"].T).view(T, H, dk), eps))
     k = rnd(unit_rms(rnd(n @ W["k"].T).view(T, G, dk), eps))
     v = rnd(n @ W["v"].T).view(T, G, dv)
@@ -131,11 +131,18 @@ def route(n, router, bias, top):
     return order, torch.softmax(torch.gather(z, 1, order), -1), z
 
 
-def experts(n, W, spec, rnd=_same, route_input=None):
-    """Weighted sum of the chosen experts' outputs plus the shared expert (where there is one)."""
+def experts(n, W, spec, rnd=_same, margins_out=None):
+    """Weighted sum of the chosen experts' outputs plus the shared expert (where there is one).
+    margins_out: a list that receives, per token, how far the last chosen logit lies above the first one left
+    out, as a share of the root mean square of all the sequence's logits about their mean (with two experts a
+    token's own spread is the margin itself); infinite where all experts are chosen."""
     E, top = spec["router"]["experts"], spec["router"]["top"]
     limit = spec["expert"]["limit"]
-    ids, wts, _ = route(n if route_input is None else route_input, W["router"], W["router.b"], top)
+    ids, wts, z = route(n, W["router"], W["router.b"], top)
+    if margins_out is not None:
+        zs = torch.sort(z, dim=-1, descending=True).values
+        spread = (z - z.mean()).pow(2).mean().sqrt().clamp_min(1e-30)
+        margins_out.append((zs[:, top - 1] - zs[:, top]) / spread if top < E else torch.full((n.shape[0],), math.inf, dtype=n.dtype))
     out = torch.zeros(n.shape[0], W["e0.down"].shape[0], dtype=n.dtype)
     for t in range(n.shape[0]):
         for j in range(top):
@@ -169,21 +176,35 @@ def hyper_step(xs, hc, fn, norm_w, eps, rnd=_same):
     return torch.einsum("sr,std->rtd", hc["mix"], xs) + hc["out"][:, None, None] * y[None]
 
 
-def forward(cfg, weights, tokens, rnd=_same, layer_outputs=None):
-    """Logits [T, vocab] of a whole sequence.  weights: float64 tensors by checkpoint name.
-    layer_outputs: a list that receives the sum of the streams after every layer run."""
+def plain_step(x, fn, norm_w, eps, rnd=_same):
+    """One sublayer over a single residual stream: x <- x + fn(norm(x))."""
+    return x + fn(rnd(offset_norm(x, norm_w, eps)))
+
+
+def forward(cfg, weights, tokens, rnd=_same, layer_outputs=None, margins_out=None):
+    """Logits [T, vocab] of a whole sequence.  weights: tensors by checkpoint name (any float type).
+    layer_outputs: a list that receives the residual stream (the sum of the streams) after every layer run.
+    margins_out: see experts().  Without 'streams' in the configuration the model keeps one stream and adds."""
+    weights = {k: v.to(F64) for k, v in weights.items()}
     eps = cfg["norm"]["eps"]
-    S = cfg.get("streams", 1)
+    S = cfg.get("streams")
     x = weights["embed"][torch.as_tensor(tokens, dtype=torch.long)]
-    xs = torch.stack([x] * S)
+    xs = x if S is None else torch.stack([x] * S)
     for i in layer_order(cfg):
         layer, W = cfg["layers"][i], sub(weights, f"l{i}.")
         m = layer["mixer"]
         attend = window_attention if layer["type"] == "attention" else latent_attention
-        xs = hyper_step(xs, sub(W, "hc1."), lambda h: attend(h, sub(W, "mix."), m, eps, rnd), W["norm1"], eps, rnd)
-        if layer.get("mlp") is not None:
-            xs = hyper_step(xs, sub(W, "hc2."), lambda h: experts(h, sub(W, "mlp."), layer["mlp"], rnd), W["norm2"], eps, rnd)
+        mix = lambda h: attend(h, sub(W, "mix."), m, eps, rnd)
+        ff = lambda h: experts(h, sub(W, "mlp."), layer["mlp"], rnd, margins_out)
+        if S is None:
+            xs = plain_step(xs, mix, W["norm1"], eps, rnd)
+            if layer.get("mlp") is not None:
+                xs = plain_step(xs, ff, W["norm2"], eps, rnd)
+        else:
+            xs = hyper_step(xs, sub(W, "hc1."), mix, W["norm1"], eps, rnd)
+            if layer.get("mlp") is not None:
+                xs = hyper_step(xs, sub(W, "hc2."), ff, W["norm2"], eps, rnd)
         if layer_outputs is not None:
-            layer_outputs.append(xs.sum(0))
-    x = xs.sum(0)
+            layer_outputs.append(xs if S is None else xs.sum(0))
+    x = xs if S is None else xs.sum(0)
     return rnd(offset_norm(x, weights["final.norm"], eps)) @ weights["head"].T

@@ -1,0 +1,406 @@
+"""Kugalorn on the GPU against the plain implementation (tests/plain/kugalorn_plain.py): every mechanism
+alone, whole prompts against token-by-token decoding, portions down to two tokens, batches of unequal
+requests, pages and slots used again, keys just inside and just outside a window in prompts and in decoding,
+far keys and page borders, first tokens, long decoding past a window, sizes nobody tuned the kernels for,
+and greedy generation through the scheduler, the command line and the trace runner."""
+import functools
+import math
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import kugalorn_util as ku
+import util
+from plain import kugalorn_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+WHOLE = ["mixed", "wide", "odd", "plain"]
+
+
+@functools.lru_cache(maxsize=None)
+def model(name: str, seed: int = 0):
+    raw = ku.CONFIGS[name]
+    w = ku.make_weights(raw, seed)
+    folder = os.path.join(util._TMP.name, f"kugalorn_{name}_{seed}")
+    return ku.write_folder(raw, w, folder), raw, w
+
+
+@functools.lru_cache(maxsize=512)
+def _plain(name, seed, tokens, scale):
+    _, raw, w = model(name, seed)
+    if scale is None:
+        return plain.forward(raw, w, list(tokens))
+    return plain.forward(raw, w, list(tokens), rnd=lambda t: plain.bf16_round(t * scale) / scale)
+
+
+CLOSE_CALL = 0.05       # of the router logits' spread: below it, bfloat16 rounding may choose another expert
+
+
+@functools.lru_cache(maxsize=512)
+def rows_before_a_close_call(name, seed, tokens) -> int:
+    _, raw, w = model(name, seed)
+    margins = []
+    plain.forward(raw, w, list(tokens), margins_out=margins)
+    n = len(tokens)
+    for m in margins:
+        close = torch.nonzero(m < CLOSE_CALL)
+        if len(close):
+            n = min(n, int(close[0]))
+    return n
+
+
+def expected(name, tokens, seed=0) -> util.Expected:
+    tokens = tuple(tokens)
+    return util.Expected(_plain(name, seed, tokens, None), [_plain(name, seed, tokens, s) for s in util.REALIZATION_SCALES])
+
+
+def engine(name, dtype, seed=0, **kw):
+    from tuff_amd.engine.engine import Engine
+    folder, _, _ = model(name, seed)
+    kw.setdefault("page_size", 16)
+    kw.setdefault("max_tokens", 1024)
+    kw.setdefault("max_requests", 4)
+    return Engine.from_folder(folder, dtype=dtype, poison_cache=True, **kw)
+
+
+def requests(name, lengths, seed=0):
+    V = ku.CONFIGS[name]["vocab"]
+    return {f"r{i}": util.rand_tokens(n, V, seed * 100 + i) for i, n in enumerate(lengths)}
+
+
+def check(name, dtype, plan, reqs, seed=0, **kw):
+    eng = engine(name, dtype, seed, **kw)
+    got = util.run_plan(eng, plan)
+    eng.manager.check()
+    assert not eng.manager.live()
+    compare(name, dtype, got, reqs, seed)
+    return eng, got
+
+
+def compare(name, dtype, got, reqs, seed=0, what=""):
+    """float32: every request against the exact logits.  bfloat16: the rows of all requests together against the
+    rounding model's error, each request up to its first token at which a router's choice hangs on less than
+    rounding moves (float32 covers the rest)."""
+    exp = {rid: expected(name, toks, seed) for rid, toks in reqs.items()}
+    if dtype == "float32":
+        for rid in reqs:
+            util.assert_close_f32(got[rid], exp[rid], f"{what} {name} {rid}")
+        return
+    rids = list(reqs)
+    keep = {r: rows_before_a_close_call(name, seed, tuple(reqs[r])) for r in rids}
+    for r in rids:
+        assert torch.isfinite(got[r]).all(), f"{what} {name} {r}: non-finite logits"
+    if sum(keep.values()) < 8:
+        return
+    want = util.Expected(torch.cat([exp[r].want[:keep[r]] for r in rids]),
+                         [torch.cat([exp[r].rounded[i][:keep[r]] for r in rids]) for i in range(len(util.REALIZATION_SCALES))])
+    util.assert_close_bf16(torch.cat([got[r][:keep[r]] for r in rids]), want, f"{what} {name} bfloat16")
+
+
+def all_single(reqs):
+    return util.plan_tail(reqs, tail=10 ** 6)
+
+
+# ------------------------------------------------------------------------ mechanisms alone
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", [n for n in ku.CONFIGS if n.startswith("only_")])
+def test_each_mechanism_alone(gpu, name, dtype):
+    reqs = requests(name, [37, 1, 9])
+    check(name, dtype, util.plan_whole(reqs), reqs)
+    check(name, dtype, util.plan_chunks(reqs, sizes=(2, 5, 1, 3, 16, 2)), reqs)
+
+
+# -------------------------------------------------------------- whole models under every plan
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", WHOLE)
+def test_whole_prompts(gpu, name, dtype):
+    reqs = requests(name, [90, 1, 2, 33])
+    check(name, dtype, util.plan_whole(reqs), reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", WHOLE)
+def test_prompt_then_single_tokens_and_single_tokens_from_the_start(gpu, name, dtype):
+    reqs = requests(name, [70, 40], seed=1)
+    check(name, dtype, util.plan_tail(reqs, tail=32), reqs, seed=1)
+    first = requests(name, [24], seed=2)                 # the first tokens of a sequence, one by one
+    check(name, dtype, all_single(first), first, seed=1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", WHOLE)
+def test_portions_of_changing_size(gpu, name, dtype):
+    reqs = requests(name, [150, 61], seed=3)
+    check(name, dtype, util.plan_chunks(reqs), reqs)
+    small = {"r1": reqs["r1"]}
+    check(name, dtype, util.plan_chunks(small, sizes=(2, 2, 3, 2, 1, 2)), small)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["mixed", "wide", "odd"])
+def test_batches_of_unequal_requests_with_pages_and_slots_used_again(gpu, name, dtype):
+    reqs = requests(name, [5, 77, 130, 2, 40, 64, 19, 95, 33], seed=4)
+    plan = util.plan_mixed(reqs, seed=4, max_live=3)
+    peak = util.live_tokens_peak(plan)
+    eng, got = check(name, dtype, plan, reqs, max_tokens=peak, max_requests=3)
+    for g in eng.manager.groups:
+        assert g.pool.allocations > g.pool.num_pages       # pages came back and went out again, in every group
+    again = util.run_plan(eng, plan)                       # every page has been used before and holds NaN now
+    if dtype == "float32":
+        for rid in reqs:
+            assert torch.equal(again[rid], got[rid]), rid
+    else:
+        compare(name, dtype, again, reqs, what="second run")
+
+
+@pytest.mark.parametrize("name", ["mixed", "odd"])
+def test_float32_logits_do_not_depend_on_the_plan(gpu, name):
+    """The same bits whether a prompt comes whole, in portions, token by token or beside other requests, with
+    recorded steps or without."""
+    reqs = requests(name, [83, 30, 47], seed=5)
+    plans = [util.plan_whole(reqs), util.plan_chunks(reqs), all_single(reqs), util.plan_mixed(reqs, seed=1)]
+    base = util.run_plan(engine(name, "float32"), plans[0])
+    for i, plan in enumerate(plans[1:]):
+        for graphs in (True, False):
+            got = util.run_plan(engine(name, "float32", use_graphs=graphs), plan)
+            for rid in reqs:
+                assert torch.equal(got[rid], base[rid]), f"plan {i + 1}, graphs {graphs}, {rid}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding_past_the_windows(gpu, dtype):
+    """Windows of 20 and 7 pass over decoded tokens many times; their pages go back to the pool on the way."""
+    reqs = requests("mixed", [330], seed=6)
+    eng, _ = check("mixed", dtype, util.plan_tail(reqs, tail=325), reqs)
+    assert eng.graph_replays > 0                           # steps of single tokens were recorded and replayed
+
+
+def test_steps_of_portions_recorded_in_sections(gpu):
+    reqs = requests("mixed", [96, 96, 96, 96], seed=7)
+    plan = util.plan_chunks(reqs, sizes=(8,))
+    eng, _ = check("mixed", "float32", plan, reqs)
+    assert eng.section_replays > 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_peaky_attention_far_keys_in_prompts_and_in_decoding(gpu, dtype):
+    """Large score scales: a few keys hold the weight, anywhere in hundreds (latent attention) or anywhere in the
+    window; a key lost, taken twice or read from a neighbour's page moves the logits."""
+    for name in ("only_latent", "only_latent_wide", "only_attention_equal", "only_attention_unmasked"):
+        reqs = requests(name, [420, 300], seed=8)
+        check(name, dtype, util.plan_tail(reqs, tail=70), reqs)
+        check(name, dtype, util.plan_chunks(reqs, sizes=(15, 1, 16, 17, 2, 31, 33, 64, 63, 65)), reqs)
+
+
+# ------------------------------------------------------------ one key made to stand out
+def _bound_attention(gpu, dtype, H, G, dk, dv, window, scale):
+    """An attention mixer whose projections are the identity: a row of its input is q | k | v."""
+    from tuff_amd.parts.attention import AttentionMixer
+    from tuff_amd.parts.base import Runtime
+    from tuff_amd.parts.linear import Linear
+    width = H * dk + G * dk + G * dv
+    mixer = AttentionMixer(width, H, G, dk, value_dim=dv, scale=scale, qk_norm_eps=1e-6, window=window, slope_span=8.0,
+                           names={k: k for k in ("q", "k", "v", "o")})
+    mixer.out = Linear("o", H * dv, H * dv)
+    eye = torch.eye(width)
+    weights = {"q": eye[:H * dk], "k": eye[H * dk:H * dk + G * dk], "v": eye[H * dk + G * dk:], "o": torch.eye(H * dv)}
+    mixer.bind({n: t.to(dtype).to(gpu) for n, t in weights.items()}, Runtime(gpu, dtype))
+    m = dict(heads=H, kv_heads=G, dim=dk, vdim=dv, scale=scale, mask={"size": window} if window else None)
+    W = {n: t.to(dtype).double() for n, t in weights.items()}
+    return mixer, width, m, W
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dk, dv, H, G, window", [(16, 16, 4, 2, 40), (64, 64, 8, 2, 300), (24, 40, 3, 1, 17), (128, 128, 2, 2, 256),
+                                                 (32, 32, 24, 1, 64), (48, 48, 2, 1, None), (8, 8, 1, 1, 1)])
+def test_window_attention_one_key_stands_out(gpu, dk, dv, H, G, window, dtype):
+    """One key is lined up with the last query's heads so that it would hold nearly all the weight, and placed just
+    inside the window, just outside it, at a page's border, at the start, far back; the last query sees it from a
+    prompt's portion and as a single token.  Pages are scattered and everything else in the pool is NaN."""
+    from tuff_amd.cache.manager import CacheLayout, CacheManager
+    from tuff_amd.cache.storage import CacheStorage
+    from tuff_amd.engine.batch import StepEntry, build_context
+    ps, scale = 16, 12.0 / dk
+    mixer, width, m, W = _bound_attention(gpu, dtype, H, G, dk, dv, window, scale)
+    gen = torch.Generator().manual_seed(dk + dv + (window or 0))
+    layout = CacheLayout.from_specs({0: mixer.cache_spec()})
+    tol = 1e-5 if dtype == torch.float32 else 2.5e-2
+    for n in (1, 17, 130, 257, 700):
+        w = window or n
+        places = {n - 1, max(0, n - w), max(0, n - w - 1), 0, (n - 1) // 16 * 16, max(0, (n - 1) // 16 * 16 - 1), n // 2}
+        for special in sorted(places):
+            mgr = CacheManager(layout, ps, 64, 2)
+            store = CacheStorage(mgr, dtype, gpu, poison=True)
+            mgr.admit("pad")
+            mgr.extend("pad", 40)                               # the request's pages do not start at page 0
+            mgr.admit("a")
+            x = torch.randn(n, width, generator=gen) * 0.5
+            krows = x[:, H * dk:H * dk + G * dk].view(n, G, dk)
+            for g in range(G):                                   # the special key lines up with the last query's heads
+                krows[special, g] = x[n - 1, :H * dk].view(H, dk)[g * (H // G)]
+            x = x.to(dtype)
+            want = plain.window_attention(x.double(), W, m, 1e-6)
+            for tail in (0, min(3, n - 1)):                      # the last query in a portion, and as a single token
+                steps = [list(range(0, n - tail))] + [[i] for i in range(n - tail, n)]
+                mgr.truncate("a", 0)
+                for rows in steps:
+                    mgr.extend("a", len(rows))
+                    ctx = build_context([StepEntry("a", [0] * len(rows), [])], mgr, gpu, 10)
+                    res = torch.zeros(len(rows), H * dv, dtype=torch.float32, device=gpu)
+                    mixer.forward(x[rows].to(gpu).contiguous(), ctx, store.views[0], res)
+                    got = res.double().cpu()
+                    err = (got - want[rows]).abs().max()
+                    assert err <= tol * max(1.0, float(want.abs().max())), (n, special, tail, rows[0], float(err))
+
+
+# ----------------------------------------------------------------------- kernels alone
+@pytest.mark.parametrize("S, d", [(1, 24), (3, 200), (8, 52), (2, 1024)])
+def test_streams_kernel_alone(gpu, S, d):
+    from tuff_amd.csrc import ops
+    g = torch.Generator().manual_seed(S * d)
+    T, eps = 11, 1e-3
+    xs, y = torch.randn(S, T, d, generator=g), torch.randn(T, d, generator=g)
+    mix, out_w, in_w, nw = torch.randn(S, S, generator=g), torch.randn(S, generator=g), torch.randn(S, generator=g), torch.randn(d, generator=g)
+    new = torch.einsum("sr,std->rtd", mix.double(), xs.double()) + out_w.double()[:, None, None] * y.double()[None]
+    u = torch.einsum("s,std->td", in_w.double(), new)
+    want_h = plain.unit_rms(u, eps) * nw.double()
+    dev = lambda t: t.to(gpu).contiguous()
+    for dt in (torch.float32, torch.bfloat16):
+        x1, h = dev(xs), torch.empty(T, d, dtype=dt, device=gpu)
+        ops.hc_step(x1, y=dev(y), mix=dev(mix), out_w=dev(out_w), in_w=dev(in_w), norm_w=dev(nw), eps=eps, h_out=h)
+        assert (x1.double().cpu() - new).abs().max() < 1e-4
+        assert (h.double().cpu() - want_h).abs().max() < (1e-4 if dt == torch.float32 else 5e-2)
+    x2, uo = dev(xs), torch.empty(T, d, device=gpu)
+    ops.hc_step(x2, in_w=dev(in_w), u_out=uo)                                 # a read alone leaves the streams as they are
+    assert torch.equal(x2.cpu(), xs) and (uo.double().cpu() - torch.einsum("s,std->td", in_w.double(), xs.double())).abs().max() < 1e-4
+    x3 = dev(xs)
+    ops.hc_step(x3, y=dev(y), mix=dev(mix), out_w=dev(out_w))                 # a write alone
+    assert (x3.double().cpu() - new).abs().max() < 1e-4
+
+
+@pytest.mark.parametrize("d, F, E, top", [(64, 40, 4, 2), (44, 20, 3, 3), (128, 256, 16, 1)])
+def test_gated_experts_both_kernels_and_the_router(gpu, d, F, E, top):
+    """The experts' kernel for any size and the matrix-core kernel against the plain clamped expert; the router's
+    bias and its softmax over the chosen logits, with ties."""
+    from tuff_amd.csrc import ops
+    g = torch.Generator().manual_seed(d + F)
+    T, limit = 70, 0.8
+    rb = lambda *s: (torch.randn(*s, generator=g) / math.sqrt(s[-1])).to(torch.bfloat16)
+    h = torch.randn(T, d, generator=g).to(torch.bfloat16)
+    gates, ups, downs = [rb(F, d) for _ in range(E)], [rb(F, d) for _ in range(E)], [rb(d, F) for _ in range(E)]
+    router, bias = torch.randn(E, d, generator=g) / math.sqrt(d), torch.randn(E, generator=g)
+    bias[1] = bias[0]
+    router[1] = router[0]                                     # experts 0 and 1 tie on every token
+    ids, wts, z = plain.route(h.double(), router.double(), bias.double(), top)
+    want = torch.zeros(T, d, dtype=torch.float64)
+    for t in range(T):
+        for j in range(top):
+            e = int(ids[t, j])
+            want[t] += wts[t, j] * plain.clamped_expert(h[t:t + 1].double(), gates[e].double(), ups[e].double(), downs[e].double(),
+                                                        limit, plain.bf16_round)[0]
+    dev = lambda t: t.to(gpu).contiguous()
+    zg, idg, wtg = torch.empty(T, E, device=gpu), torch.empty(T, top, dtype=torch.int32, device=gpu), torch.empty(T, top, device=gpu)
+    ops.moe_router(dev(h), dev(router), zg, idg, wtg, E=E, top=top, weights="softmax", bias=dev(bias))
+    assert (zg.double().cpu() - z).abs().max() < 1e-4
+    zs = torch.sort(z, -1, descending=True).values
+    gaps = (zs[:, :-1] - zs[:, 1:])[:, :top if top < E else E - 1]       # between neighbours in the order, down to the border
+    firm = ((gaps > 1e-3) | (gaps == 0)).all(1)                          # (an exact tie is decided by the index, in both)
+    assert firm.sum() > T // 2
+    assert torch.equal(idg.cpu()[firm].long(), ids[firm]) and (wtg.double().cpu()[firm] - wts[firm]).abs().max() < 1e-5
+    both = (idg.cpu() == 0).any(1) & (idg.cpu() == 1).any(1)
+    for row in idg.cpu()[both].tolist():
+        assert row.index(0) + 1 == row.index(1)               # the lower index of a tie comes first
+    form = dict(activation="swish_clamp", scale_input=False, gated=True, limit=limit, alpha=1.702)
+    idp, wtp = dev(ids.to(torch.int32)), dev(wts.float())
+    res = torch.zeros(T, d, device=gpu)
+    ops.moe_experts(dev(h), dev(torch.stack([torch.cat([a, b]) for a, b in zip(gates, ups)])), dev(torch.stack(downs)), idp, wtp, res, **form)
+    assert (res.double().cpu() - want).abs().max() < 2e-2 * max(1.0, float(want.abs().max()))
+    if ops.moe_grouped_supported(torch.bfloat16, d, F, E):
+        res2 = torch.zeros(T, d, device=gpu)
+        ops.moe_experts_grouped(dev(h), ops.tile_experts([dev(ops.interleave_gate_up(a, b)) for a, b in zip(gates, ups)]),
+                                ops.tile_experts([dev(w) for w in downs]), idp, wtp, res2, F=F, **form)
+        assert (res2.double().cpu() - want).abs().max() < 2e-2 * max(1.0, float(want.abs().max()))
+        assert (res2 - res).abs().max() < 1e-2 * max(1.0, float(want.abs().max()))
+
+
+def test_latent_kernels_alone(gpu):
+    """Norm, rotation of neighbouring pairs with fewer channels turning than the part holds, the cache row, and
+    the per-head products with and without the gate, float32, against the plain functions."""
+    from tuff_amd.csrc import ops
+    g = torch.Generator().manual_seed(9)
+    T, H, dk, dr, rank, dims, ps = 37, 3, 10, 6, 20, 4, 16
+    lat = rank + dr
+    width = H * (dk + dr) + lat + H
+    proj = torch.randn(T, width, generator=g)
+    nw = 1 + 0.3 * torch.randn(rank, generator=g)
+    pos = torch.arange(100, 100 + T)
+    inv_freq = torch.tensor([50.0 ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=torch.float64).float()
+    slots = torch.randperm(4 * ps, generator=g)[:T].to(torch.int32)
+    cache = torch.full((4, 1, ps, lat), float("nan"), device=gpu)
+    q_lat = torch.zeros(T, H * lat, device=gpu)
+    dev = lambda t: t.to(gpu).contiguous()
+    ops.latent_post(dev(proj), q_lat, cache, q_off=0, ckr_off=H * (dk + dr), norm_w=dev(nw), eps=1e-4, inv_freq=dev(inv_freq),
+                    rot_dims=dims, positions=dev(pos.to(torch.int32)), slot_mapping=dev(slots), H=H, dim=dk, rot=dr, rank=rank)
+    ckr = proj[:, H * (dk + dr):H * (dk + dr) + lat].double()
+    rows = torch.cat([plain.plain_norm(ckr[:, :rank], nw.double(), 1e-4), plain.rotate_pairs(ckr[:, rank:], pos, 50.0, dims)], 1)
+    got_rows = cache.view(-1, lat)[slots.long().to(gpu)].double().cpu()
+    assert (got_rows - rows).abs().max() < 2e-4          # float32 angles at positions of a hundred
+    q = proj[:, :H * (dk + dr)].view(T, H, dk + dr).double()
+    want_rot = plain.rotate_pairs(q[..., dk:], pos, 50.0, dims)
+    assert (q_lat.view(T, H, lat)[..., rank:].double().cpu() - want_rot).abs().max() < 2e-4
+    w_uk = torch.randn(H, dk, rank, generator=g)
+    ops.head_matmul(dev(proj), dev(w_uk), q_lat, H=H, x_head=dk + dr, y_head=lat)
+    assert (q_lat.view(T, H, lat)[..., :rank].double().cpu() - torch.einsum("thk,hkn->thn", q[..., :dk], w_uk.double())).abs().max() < 1e-4
+    assert (q_lat.view(T, H, lat)[..., rank:].double().cpu() - want_rot).abs().max() < 2e-4       # the rotated parts stay
+    out = torch.zeros(T, H * 5, device=gpu)
+    w_uv = torch.randn(H, rank, 5, generator=g)
+    x = torch.randn(T, H * rank, generator=g)
+    ops.head_matmul(dev(x), dev(w_uv), out, H=H, x_head=rank, y_head=5, gate=dev(proj), gate_col=width - H)
+    want = torch.einsum("thk,hkn->thn", x.view(T, H, rank).double(), w_uv.double()) * torch.sigmoid(proj[:, width - H:].double())[..., None]
+    assert (out.view(T, H, 5).double().cpu() - want).abs().max() < 1e-4
+
+
+# ------------------------------------------------------------------- generation, command line
+def _plain_greedy(name, prompt, n_new, seed=0):
+    _, raw, w = model(name, seed)
+    toks = list(prompt)
+    for _ in range(n_new):
+        toks.append(int(plain.forward(raw, w, toks)[-1].argmax()))
+    return toks[len(prompt):]
+
+
+def test_greedy_generation_through_the_scheduler(gpu):
+    from tuff_amd.engine.llm import LLM
+    from tuff_amd.sampling.params import SamplingParams
+    reqs = requests("mixed", [5, 21, 1, 12, 30, 8], seed=9)
+    eng = engine("mixed", "float32", max_tokens=512, max_requests=3)
+    llm = LLM(engine=eng, max_num_seqs=3, max_batched_tokens=16, ctx_size=128, ignore_eos=True)
+    outs = llm.generate(list(reqs.values()), SamplingParams(temp=0.0, max_new_tokens=10, ignore_eos=True))
+    for g, prompt in zip(outs, reqs.values()):
+        assert list(g.token_ids) == _plain_greedy("mixed", prompt, 10), prompt
+    eng.manager.check()
+    assert not eng.manager.live()
+
+
+def test_command_line_and_trace_replay(gpu, tmp_path):
+    folder, raw, _ = model("wide")
+    prompt = util.rand_tokens(9, raw["vocab"], 3)
+    p = subprocess.run([sys.executable, os.path.join(util.ROOT, "bin", "tuff"), "--model", folder, "--prompt-ids",
+                        ",".join(map(str, prompt)), "--dump-tokens", "-n", "6", "--dtype", "fp32", "--temp", "0"],
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [int(x) for x in p.stdout.split()] == _plain_greedy("wide", prompt, 6)
+    q = subprocess.run([sys.executable, os.path.join(util.ROOT, "bin", "tuff"), "--model", folder, "--inspect"],
+                       capture_output=True, text=True, timeout=300)
+    assert q.returncode == 0 and "LatentAttentionMixer" in q.stdout and "HyperConnectionBlock" in q.stdout, q.stdout[-2000:] + q.stderr[-2000:]
+    # the trace runner: a mixed plan through a child process, four slots, a pool no larger than the plan's peak
+    reqs = requests("wide", [50, 3, 70, 20, 31], seed=10)
+    plan = util.plan_mixed(reqs, seed=2)
+    for dtype in DTYPES:
+        got = util.run_trace_run(folder, dtype, plan, util.live_tokens_peak(plan), str(tmp_path / dtype))
+        compare("wide", dtype, got, reqs, what="trace runner")

@@ -304,7 +304,8 @@ def run_trace_run(model_dir: str, dtype: str, plan, max_tokens: int, out_dir: st
         if proc.poll() is None:
             proc.kill()
     with open(os.path.join(model_dir, "config.json")) as f:
-        V = json.load(f)["vocab_size"]
+        raw = json.load(f)
+        V = raw["vocab_size"] if "vocab_size" in raw else raw["vocab"]
     fed, rows = {}, {}
     for s in plan:
         n_want = sum(len(e["want"]) for e in s["entries"])

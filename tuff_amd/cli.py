@@ -86,7 +86,7 @@ def _inspect(cfg, model, out=sys.stdout) -> None:
         mixer, ffn = getattr(b, "mixer", None), getattr(b, "ffn", None)
         inside = " + ".join(type(p).__name__ for p in (mixer, ffn) if p is not None) or type(b).__name__
         spec = mixer.cache_spec() if hasattr(mixer, "cache_spec") else None
-        print(f"  layer {i}: {inside}  cache: {spec}", file=out)
+        print(f"  layer {i}: {type(b).__name__}: {inside}  cache: {spec}", file=out)
     print(f"run order: {[r.block for r in model.schedule]}", file=out)
 
 
