@@ -53,6 +53,9 @@ struct FusedQKV {
     const float* angles = nullptr;         // [n_angles][2][32]: cosines and sines of pos * inv_freq, or null
     int n_angles = 0;
     const int* slot_mapping = nullptr;     // [tokens]; null: the cache is only read
+    // (not of the fused form, but of every form: it travels here)  A distance slope per head [H], or null:
+    // slopes[h] * (position - key) is taken off head h's scaled scores.
+    const float* slopes = nullptr;
 };
 
 // cosine and sine of pos * inv_freq[j]: from the table where it reaches, else computed (the same bits)
@@ -296,6 +299,8 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
 
     // this lane's columns
     int pos_c[NB], lo_c[NB];
+    float slope_c[NB];
+    const bool has_slopes = fq.slopes != nullptr;
     long long qrow[NB];                    // row of the column in the work space; -1: no column
     bf16x8 qf[NB][KC];
 #pragma unroll
@@ -304,6 +309,7 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
         const bool valid = c < ncols;
         const int tok = t0 + (valid ? c / G : 0);
         const int head = kvh * G + (valid ? c % G : 0);
+        slope_c[nb] = has_slopes ? fq.slopes[head] : 0.f;
         pos_c[nb] = valid ? pos0 + c / G : -1;
         lo_c[nb] = (valid && window > 0) ? max(0, pos_c[nb] - window + 1) : 0;
         qrow[nb] = valid ? (long long)tok * H + head : -1;
@@ -398,7 +404,9 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
                 for (int e = 0; e < 4; ++e) {
                     const int key = key0 + 8 * g + 4 * kb + e;
                     const bool ok = my_live && key <= pos_c[nb] && key >= lo_c[nb];
-                    const float x = ok ? s[kb][nb][e] * scale : -INFINITY;
+                    // (the distance as an integer first: far positions lose no bits)
+                    const float x = !ok ? -INFINITY : has_slopes ? fmaf(s[kb][nb][e], scale, slope_c[nb] * (float)(key - pos_c[nb]))
+                                                                  : s[kb][nb][e] * scale;
                     v[kb * 4 + e] = x;
                     mx = fmaxf(mx, x);
                 }
@@ -782,7 +790,7 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
                             float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
                             const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
                             int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
-                            int n_parts, hipStream_t stream, const float* sinks = nullptr) {
+                            int n_parts, hipStream_t stream, const float* sinks = nullptr, const float* slopes = nullptr) {
     if (n_tokens <= 0 || n_qblocks <= 0) return 0;
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0 || n_parts < 1) return -2;
     if (Hkv > 65535 || n_qblocks > 65535 || n_parts > COMBINE_MAX_PARTS) return -2;
@@ -790,8 +798,10 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
     bf16_t* K = (bf16_t*)k_cache;                                        // read only without the fused form
     bf16_t* V = (bf16_t*)v_cache;
     dim3 grid(n_parts, n_qblocks, Hkv);
+    FusedQKV plain_form;
+    plain_form.slopes = slopes;
 #define GO(HDP, NB) launch_partition<HDP, NB, false>(grid, stream, Q, K, V, ws_o, ws_ml, block_table, max_blocks, (const int2*)blk, \
-                                                     (const int4*)req_info, H, Hkv, hd, page_size, window, scale, n_parts, FusedQKV())
+                                                     (const int4*)req_info, H, Hkv, hd, page_size, window, scale, n_parts, plain_form)
 #define BY_NB(HDP) do { if (nb == 1) GO(HDP, 1); else if (nb == 2) GO(HDP, 2); else if (nb == 4) GO(HDP, 4); else return -2; } while (0)
     if (hd <= 32) BY_NB(32);
     else if (hd <= 64) BY_NB(64);
@@ -804,6 +814,17 @@ static int launch_attention(const void* q, const void* k_cache, const void* v_ca
     if (rc) return rc;
     return launch_merge((const float*)ws_o, (const float*)ws_ml, (bf16_t*)out, positions, n_tokens, H, hd, window, n_parts, PART,
                         stream, sinks);
+}
+
+// The same with a sink per head and a distance slope per head (each float32 [H], or null): slopes[h] * (position - key)
+// is taken off head h's scaled scores.
+TUFF_EXPORT int tuff_attention_mfma_biased(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                           float* ws_o, float* ws_ml, const int* block_table, int max_blocks,
+                                           const int* blk, int n_qblocks, int nb, const int* req_info, const int* positions,
+                                           int n_tokens, int H, int Hkv, int hd, int page_size, int window, float scale,
+                                           int n_parts, const float* sinks, const float* slopes, hipStream_t stream) {
+    return launch_attention(q, k_cache, v_cache, out, ws_o, ws_ml, block_table, max_blocks, blk, n_qblocks, nb, req_info,
+                            positions, n_tokens, H, Hkv, hd, page_size, window, scale, n_parts, stream, sinks, slopes);
 }
 
 // The number of lanes of a wave that fetch page numbers for partition `part` with pages of page_size

@@ -48,7 +48,8 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     bf16_t* __restrict__ out, const int* __restrict__ block_table, int max_blocks,
     const int2* __restrict__ blk, const int4* __restrict__ req_info,
     int H, int Hkv, int hd, int page_size, int window, float scale_log2e,
-    int seg_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml, const float* __restrict__ sinks) {
+    int seg_keys, float* __restrict__ ws_o, float* __restrict__ ws_ml, const float* __restrict__ sinks,
+    const float* __restrict__ slopes) {
     constexpr int KC = HDP / 32;          // 32-wide chunks of the head dimension
     constexpr int DB = HDP / 16;          // 16-wide blocks of output channels
     constexpr int HC = HDP / 8;           // 16-byte chunks of a K row
@@ -89,6 +90,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
     // ---- this wave's columns
     const int wcol0 = col0 + wave * NBW * 16;
     int pos_c[NBW], lo_c[NBW];
+    float slope_c[NBW];                    // the head's distance slope, in base-2 exponents; 0: none
     long long qrow[NBW];                   // row of the column in q and out; -1: no column
     bf16x8 qf[NBW][KC];
     int wave_pos_max = -1, wave_pos_min = 0x7fffffff, wave_lo_max = 0;
@@ -98,6 +100,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
         const bool valid = c < ncols;
         const int tok = t0 + (valid ? c / G : 0);
         const int head = kvh * G + (valid ? c % G : 0);
+        slope_c[nb] = slopes ? slopes[head] * 1.4426950408889634f : 0.f;
         pos_c[nb] = valid ? pos0 + c / G : -1;
         lo_c[nb] = (valid && window > 0) ? max(0, pos_c[nb] - window + 1) : 0;
         qrow[nb] = valid ? (long long)tok * H + head : -1;
@@ -299,6 +302,21 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             // it is the same instruction with and without the mask.
             float mx = -INFINITY;
             bool ok[2][8];
+            if (slopes) {
+                // Heads with a distance slope: slope * (position - key) is taken off the scaled score (from the
+                // integer distance, so that far positions lose no bits).  The scores become exponents here, the
+                // maximum is theirs, and the scale below is 1.
+#pragma unroll
+                for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int key = key0 + 32 * sub + 8 * g + 4 * kb + e;
+                            sc[sub].v[kb][nb][e] = fmaf(sc[sub].v[kb][nb][e], scale_log2e, slope_c[nb] * (float)(key - pos_c[nb]));
+                        }
+            }
+            const float unit = slopes ? 1.f : scale_log2e;
 #pragma unroll
             for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
@@ -315,7 +333,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             // The reference point of the exponents moves only when a score exceeds it by more than
             // 2^SLACK: until then the weights may reach 2^SLACK instead of 1, which float32 sums and
             // bfloat16 weights hold as well, and the output so far need not be rescaled.
-            const float m_cand = mx * scale_log2e;
+            const float m_cand = mx * unit;
             const float m_new = (m_cand > m_run[nb] + SLACK) ? m_cand : m_run[nb];
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
             corr[nb] = __builtin_amdgcn_exp2f(m_run[nb] - m_safe);           // 0 while nothing was seen yet
@@ -324,7 +342,7 @@ __global__ __launch_bounds__(NT) void attn_prefill_kernel(
             for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    const float p = ok[sub][i] ? __builtin_amdgcn_exp2f(fmaf(sc[sub].v[i / 4][nb][i % 4], scale_log2e, -m_safe)) : 0.f;
+                    const float p = ok[sub][i] ? __builtin_amdgcn_exp2f(fmaf(sc[sub].v[i / 4][nb][i % 4], unit, -m_safe)) : 0.f;
                     pf[sub][nb][i] = (bf16_t)p;
                 }
             m_run[nb] = m_new;
@@ -421,7 +439,7 @@ template <int HDP, int NBW, int AHEAD>
 int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, bf16_t* out,
            const int* bt, int max_blocks, const int2* blk, const int4* req_info,
            int H, int Hkv, int hd, int ps, int window, float scale_log2e, int seg_keys, float* ws_o, float* ws_ml,
-           const float* sinks) {
+           const float* sinks, const float* slopes) {
     auto kern = attn_prefill_kernel<HDP, NBW, AHEAD>;
     constexpr int lds = 2 * (STEP * (HDP + 8) + HDP * VROW) * 2;
     static bool set = false;
@@ -430,7 +448,7 @@ int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, con
         set = true;
     }
     hipLaunchKernelGGL(kern, grid, dim3(NT), lds, stream, q, kc, vc, out, bt, max_blocks, blk, req_info,
-                       H, Hkv, hd, ps, window, scale_log2e, seg_keys, ws_o, ws_ml, sinks);
+                       H, Hkv, hd, ps, window, scale_log2e, seg_keys, ws_o, ws_ml, sinks, slopes);
     return launch_status();
 }
 }  // namespace
@@ -448,11 +466,12 @@ TUFF_EXPORT int tuff_attention_prefill_block_columns(int hd) { return hd <= 128 
 // part_keys = seg_keys.
 // sinks (float32 [H], or null): a logit per head that counts once, unscaled, in the denominator and has no
 // value; with key segments it enters at the merge instead (tuff_attention_merge_sinks), not here.
-TUFF_EXPORT int tuff_attention_prefill_sinks(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                             const int* block_table, int max_blocks, const int* blk, int n_qblocks,
-                                             const int* req_info, int H, int Hkv, int hd, int page_size, int window,
-                                             float scale, int n_segs, int seg_keys, float* ws_o, float* ws_ml,
-                                             const float* sinks, hipStream_t stream) {
+// slopes (float32 [H], or null): slopes[h] * (position - key) is taken off head h's scaled scores.
+TUFF_EXPORT int tuff_attention_prefill_biased(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                              const int* block_table, int max_blocks, const int* blk, int n_qblocks,
+                                              const int* req_info, int H, int Hkv, int hd, int page_size, int window,
+                                              float scale, int n_segs, int seg_keys, float* ws_o, float* ws_ml,
+                                              const float* sinks, const float* slopes, hipStream_t stream) {
     if (n_qblocks <= 0) return 0;
     if (hd > 256 || hd % 8 != 0 || page_size % 16 != 0 || Hkv <= 0 || H % Hkv != 0) return -2;
     if (Hkv > 65535 || !(scale > 0.f)) return -2;
@@ -466,13 +485,22 @@ TUFF_EXPORT int tuff_attention_prefill_sinks(const void* q, const void* k_cache,
     dim3 grid(n_qblocks * Hkv, 1, n_segs);
     const float sl = scale * 1.4426950408889634f;
 #define GO(HDP, NBW, AHEAD) return launch<HDP, NBW, AHEAD>(grid, stream, Q, K, V, (bf16_t*)out, block_table, max_blocks, (const int2*)blk, \
-                                             (const int4*)req_info, H, Hkv, hd, page_size, window, sl, seg_keys, ws_o, ws_ml, n_segs > 1 ? nullptr : sinks)
+                                             (const int4*)req_info, H, Hkv, hd, page_size, window, sl, seg_keys, ws_o, ws_ml, n_segs > 1 ? nullptr : sinks, slopes)
     if (hd <= 32) GO(32, 2, 3);
     else if (hd <= 64) GO(64, 2, 2);
     else if (hd <= 96) GO(96, 2, 2);
     else if (hd <= 128) GO(128, 2, 2);
     else GO(256, 1, 1);
 #undef GO
+}
+
+TUFF_EXPORT int tuff_attention_prefill_sinks(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                             const int* block_table, int max_blocks, const int* blk, int n_qblocks,
+                                             const int* req_info, int H, int Hkv, int hd, int page_size, int window,
+                                             float scale, int n_segs, int seg_keys, float* ws_o, float* ws_ml,
+                                             const float* sinks, hipStream_t stream) {
+    return tuff_attention_prefill_biased(q, k_cache, v_cache, out, block_table, max_blocks, blk, n_qblocks, req_info, H, Hkv, hd,
+                                         page_size, window, scale, n_segs, seg_keys, ws_o, ws_ml, sinks, nullptr, stream);
 }
 
 TUFF_EXPORT int tuff_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,

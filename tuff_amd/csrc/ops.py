@@ -114,6 +114,9 @@ _SIGNATURES = {
         "tuff_attention_mfma_sinks": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                                       _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p],
+        "tuff_attention_mfma_biased": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                                       _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p,
+                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p],
         "tuff_attention_merge_sinks": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                        _c_void_p, _c_void_p],
         "tuff_attention_merge": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -133,6 +136,9 @@ _SIGNATURES = {
         "tuff_attention_prefill_sinks": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
                                          _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
                                          _c_void_p, _c_void_p, _c_void_p, _c_void_p],
+        "tuff_attention_prefill_biased": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int,
+                                          _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
+                                          _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
         "tuff_attention_prefill_block_columns": [_c_int],
     },
     "shortconv": {
@@ -921,14 +927,16 @@ def attention_mfma_supported(dtype, hd: int, page_size: int) -> bool:
 
 
 def attention_mfma(q, k_cache, v_cache, out, *, block_table, blocks, nb, req_info, positions,
-                   H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None, sinks=None) -> None:
+                   H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None, sinks=None, slopes=None) -> None:
     """Matrix-core attention over the paged bfloat16 cache.  blocks: int32 [n_blocks, 2] from
     query_blocks(), or None when every request's columns fit one block (block b = request b).
     req_info: int32 [R, 4] = (first token in the step, tokens, first position, -) per request.
     max_ctx_len bounds every position + 1 of the step.  sinks: float32 [H] or None, a logit per head that
-    counts once in the softmax's denominator and has no value."""
+    counts once in the softmax's denominator and has no value.  slopes: float32 [H] or None; slopes[h] * (position - key)
+    is taken off head h's scaled scores."""
     T = q.shape[0]
     _opt("sinks", sinks, torch.float32, (H,))
+    _opt("slopes", slopes, torch.float32, (H,))
     if not attention_mfma_supported(q.dtype, hd, page_size):
         raise KernelError(f"attention_mfma: needs bfloat16, a head size that is a multiple of 8 (got {hd}) "
                           f"and a page size that is a multiple of 16 (got {page_size})")
@@ -963,7 +971,10 @@ def attention_mfma(q, k_cache, v_cache, out, *, block_table, blocks, nb, req_inf
     args = (q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), ws_o.data_ptr(), ws_ml.data_ptr(),
             block_table.data_ptr(), block_table.shape[1], None if blocks is None else blocks.data_ptr(), nblk, nb,
             req_info.data_ptr(), positions.data_ptr(), T, H, Hkv, hd, page_size, int(window or 0), float(scale), n_parts)
-    if sinks is None:
+    if slopes is not None:
+        _check(load("attention_mfma").tuff_attention_mfma_biased(*args, None if sinks is None else sinks.data_ptr(), slopes.data_ptr(),
+                                                                 _stream()), "attention_mfma")
+    elif sinks is None:
         _check(load("attention_mfma").tuff_attention_mfma(*args, _stream()), "attention_mfma")
     else:
         _check(load("attention_mfma").tuff_attention_mfma_sinks(*args, sinks.data_ptr(), _stream()), "attention_mfma")
@@ -1036,7 +1047,7 @@ PREFILL_MIN_SEGMENT = 1024       # keys; shorter segments are not worth their me
 
 
 def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info,
-                      H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None, positions=None, sinks=None) -> None:
+                      H, Hkv, hd, page_size, max_ctx_len, window=0, scale=None, positions=None, sinks=None, slopes=None) -> None:
     """Matrix-core attention for steps with prompt portions: a workgroup walks over all keys of a
     block of query columns, keys and values staged through LDS; writes `out` directly.
     blocks: int32 [n_blocks, 2] from query_blocks(q_len, G, attention_prefill_block_columns(hd) // 16),
@@ -1047,6 +1058,7 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
     written, also those of tokens no block covers (with meaningless values)."""
     T = q.shape[0]
     _opt("sinks", sinks, torch.float32, (H,))      # a logit per head that counts once in the denominator and has no value
+    _opt("slopes", slopes, torch.float32, (H,))    # slopes[h] * (position - key) is taken off head h's scaled scores
     if not attention_mfma_supported(q.dtype, hd, page_size):
         raise KernelError(f"attention_prefill: needs bfloat16, a head size that is a multiple of 8 (got {hd}) "
                           f"and a page size that is a multiple of 16 (got {page_size})")
@@ -1093,7 +1105,14 @@ def attention_prefill(q, k_cache, v_cache, out, *, block_table, blocks, req_info
             None if ws_o is None else ws_o.data_ptr(), None if ws_ml is None else ws_ml.data_ptr())
     merge = (ws_o.data_ptr(), ws_ml.data_ptr(), out.data_ptr(), positions.data_ptr(), T, H, hd, int(window or 0), n_segs,
              seg_keys) if n_segs > 1 else None
-    if sinks is None:
+    if slopes is not None:
+        _check(load("attention_prefill").tuff_attention_prefill_biased(*args, None if sinks is None else sinks.data_ptr(),
+                                                                       slopes.data_ptr(), _stream()), "attention_prefill")
+        if merge is not None and sinks is None:
+            _check(load("attention_mfma").tuff_attention_merge(*merge, _stream()), "attention_merge")
+        elif merge is not None:
+            _check(load("attention_mfma").tuff_attention_merge_sinks(*merge, sinks.data_ptr(), _stream()), "attention_merge")
+    elif sinks is None:
         _check(load("attention_prefill").tuff_attention_prefill(*args, _stream()), "attention_prefill")
         if merge is not None:
             _check(load("attention_mfma").tuff_attention_merge(*merge, _stream()), "attention_merge")

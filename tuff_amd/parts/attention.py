@@ -83,9 +83,7 @@ class AttentionMixer(Mixer):
         return decls
 
     def kernel_modules(self):
-        mods = ["rope_kv", "attention"]
-        if self.slope_span is None:
-            mods += ["attention_mfma", "attention_prefill"]       # (the matrix-core kernels know no distance slopes)
+        mods = ["rope_kv", "attention", "attention_mfma", "attention_prefill"]
         if self.position is not None:
             mods += self.position.kernel_modules()
         return mods
@@ -218,10 +216,10 @@ class AttentionMixer(Mixer):
 
     def attend(self, q, o, ctx, cache, g) -> None:
         G = self.H // self.Hkv
-        if self.vd == self.hd and self.slopes is None and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
+        if self.vd == self.hd and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
             common = dict(block_table=g.block_table, req_info=ctx.req_info, H=self.H, Hkv=self.Hkv, hd=self.hd,
                           page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
-                          scale=self.scale, sinks=self.sinks)
+                          scale=self.scale, sinks=self.sinks, slopes=self.slopes)
             if ctx.max_q_len > 1:
                 # prompt portions in the step: blocks of columns walk over their keys through LDS.
                 # Requests with a single token beside them (runs of neighbours in the step's order) go
