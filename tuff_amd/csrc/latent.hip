@@ -23,7 +23,7 @@ constexpr int POST_THREADS = 256;
 template <typename T, typename TW>
 __global__ __launch_bounds__(POST_THREADS) void latent_post_kernel(
     const T* __restrict__ proj, int row_stride, int q_off, int ckr_off, T* __restrict__ q_lat, T* __restrict__ cache,
-    const TW* __restrict__ norm_w, float eps, const float* __restrict__ inv_freq, int rot_dims,
+    T* __restrict__ cache_t, int page_size, const TW* __restrict__ norm_w, float eps, const float* __restrict__ inv_freq, int rot_dims,
     const int* __restrict__ positions, const int* __restrict__ slot_mapping, int H, int dim, int rot, int rank) {
     __shared__ float scratch[POST_THREADS / WAVE];
     const long long t = blockIdx.x;
@@ -36,10 +36,17 @@ __global__ __launch_bounds__(POST_THREADS) void latent_post_kernel(
     const float total = block_sum<POST_THREADS / WAVE>(ss, scratch);
     const float inv = 1.0f / sqrtf(total / (float)rank + eps);
     const long long slot = slot_mapping ? slot_mapping[t] : -1;
+    // cache_t: the same row once more with a channel's positions contiguous within the page,
+    // [page][channel][offset], as the matrix-core attention kernels read values
+    T* dst_t = nullptr;
+    if (slot >= 0 && cache_t) dst_t = cache_t + (slot / page_size) * (long long)lat * page_size + slot % page_size;
     if (slot >= 0) {
         T* dst = cache + slot * lat;
-        for (int c = threadIdx.x; c < rank; c += POST_THREADS)
-            dst[c] = from_f32<T>(to_f32(row[ckr_off + c]) * inv * to_f32(norm_w[c]));
+        for (int c = threadIdx.x; c < rank; c += POST_THREADS) {
+            const T v = from_f32<T>(to_f32(row[ckr_off + c]) * inv * to_f32(norm_w[c]));
+            dst[c] = v;
+            if (dst_t) dst_t[(long long)c * page_size] = v;
+        }
     }
     // rotated parts: item 0 is the shared key part, items 1..H the heads' query parts; a thread a pair
     const int pairs = rot / 2, odd = rot % 2;
@@ -48,7 +55,12 @@ __global__ __launch_bounds__(POST_THREADS) void latent_post_kernel(
         const T* src = item == 0 ? row + ckr_off + rank : row + q_off + (long long)(item - 1) * (dim + rot) + dim;
         T* dst = item == 0 ? (slot >= 0 ? cache + slot * lat + rank : nullptr) : q_lat + (t * H + (item - 1)) * lat + rank;
         if (!dst) continue;
-        if (p == pairs) { dst[rot - 1] = src[rot - 1]; continue; }       // a last channel without a partner passes
+        T* dt2 = item == 0 && dst_t ? dst_t + (long long)rank * page_size : nullptr;
+        if (p == pairs) {                                                // a last channel without a partner passes
+            dst[rot - 1] = src[rot - 1];
+            if (dt2) dt2[(long long)(rot - 1) * page_size] = src[rot - 1];
+            continue;
+        }
         float u = to_f32(src[2 * p]), v = to_f32(src[2 * p + 1]);
         if (2 * p + 1 < rot_dims) {
             const float a = pos * inv_freq[p];
@@ -58,6 +70,7 @@ __global__ __launch_bounds__(POST_THREADS) void latent_post_kernel(
         }
         dst[2 * p] = from_f32<T>(u);
         dst[2 * p + 1] = from_f32<T>(v);
+        if (dt2) { dt2[(long long)(2 * p) * page_size] = from_f32<T>(u); dt2[(long long)(2 * p + 1) * page_size] = from_f32<T>(v); }
     }
 }
 
@@ -117,14 +130,17 @@ __global__ __launch_bounds__(256) void head_matmul_kernel(const T* __restrict__ 
 // channels [rank] and the shared key part [rot] from ckr_off.  Writes cache row slot_mapping[t] = [norm(c) w | rotate(k)]
 // (cache [slots][rank + rot]; slot_mapping null or a negative slot: nothing is written) and q_lat[t][h][rank ..] =
 // rotate(q_rot); q_lat [T][H][rank + rot].  norm_w [rank] of type norm_dt; inv_freq float32 [rot_dims / 2].
-TUFF_EXPORT int tuff_latent_post(const void* proj, int row_stride, int q_off, int ckr_off, void* q_lat, void* cache, int dt,
+// cache_t (or null): the rows once more as [pages][rank + rot][page_size], for kernels that read values that way.
+TUFF_EXPORT int tuff_latent_post(const void* proj, int row_stride, int q_off, int ckr_off, void* q_lat, void* cache,
+                                 void* cache_t, int page_size, int dt,
                                  const void* norm_w, int norm_dt, float eps, const float* inv_freq, int rot_dims,
                                  const int* positions, const int* slot_mapping, int n_tokens, int H, int dim, int rot, int rank,
                                  hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (H < 1 || dim < 0 || rot < 0 || rank < 1 || rot_dims < 0 || rot_dims > rot || rot_dims % 2) return -2;
+    if (cache_t && page_size < 1) return -2;
 #define LAUNCH(T, TW) hipLaunchKernelGGL((latent_post_kernel<T, TW>), dim3(n_tokens), dim3(POST_THREADS), 0, stream, (const T*)proj, \
-        row_stride, q_off, ckr_off, (T*)q_lat, (T*)cache, (const TW*)norm_w, eps, inv_freq, rot_dims, positions, slot_mapping, H, dim, rot, rank)
+        row_stride, q_off, ckr_off, (T*)q_lat, (T*)cache, (T*)cache_t, page_size, (const TW*)norm_w, eps, inv_freq, rot_dims, positions, slot_mapping, H, dim, rot, rank)
     if (dt == DT_F32 && norm_dt == DT_F32) LAUNCH(float, float);
     else if (dt == DT_F32) LAUNCH(float, bf16_t);
     else if (norm_dt == DT_F32) LAUNCH(bf16_t, float);

@@ -102,7 +102,7 @@ _SIGNATURES = {
                          _c_int, _c_int, _c_int, _c_float, _c_void_p],
     },
     "latent": {
-        "tuff_latent_post": [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_float,
+        "tuff_latent_post": [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_float,
                              _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_head_matmul": [_c_void_p, _c_ll, _c_ll, _c_void_p, _c_void_p, _c_ll, _c_ll, _c_void_p, _c_ll, _c_int,
                              _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -858,12 +858,13 @@ def hc_step(xs, *, y=None, mix=None, out_w=None, in_w=None, norm_w=None, eps: fl
 
 # ------------------------------------------------------------------- latent attention
 def latent_post(proj, q_lat, cache, *, q_off: int, ckr_off: int, norm_w, eps: float, inv_freq, rot_dims: int, positions,
-                slot_mapping, H: int, dim: int, rot: int, rank: int) -> None:
+                slot_mapping, H: int, dim: int, rot: int, rank: int, cache_t=None) -> None:
     """From a token's projected row proj[t] (queries [H, dim + rot] from column q_off; the latent's raw channels
     [rank] and the shared key part [rot] from column ckr_off): the cache row [norm(c) * norm_w | rotate(k)] at
     slot_mapping[t] (cache [pages, 1, page size, rank + rot]; slot_mapping None: no write) and the rotated query
     parts into q_lat[t, h, rank:] (q_lat [T, H * (rank + rot)]).  Rotation of neighbouring pairs of the first rot_dims
-    channels by position * inv_freq (float32 [rot_dims / 2])."""
+    channels by position * inv_freq (float32 [rot_dims / 2]).  cache_t ([pages, 1, rank + rot, page size], optional):
+    the same rows once more with a channel's positions contiguous within the page."""
     T = proj.shape[0]
     dt = proj.dtype
     lat = rank + rot
@@ -874,6 +875,7 @@ def latent_post(proj, q_lat, cache, *, q_off: int, ckr_off: int, norm_w, eps: fl
     if cache.dim() != 4 or cache.shape[1] != 1 or cache.shape[3] != lat:
         raise KernelError(f"latent_post: the cache must be [pages, 1, page size, {lat}], got {tuple(cache.shape)}")
     _gpu("cache", cache, dt)
+    _opt("cache_t", cache_t, dt, (cache.shape[0], 1, lat, cache.shape[2]))
     _gpu("norm_w", norm_w, shape=(rank,))
     if rot_dims % 2 or not 0 <= rot_dims <= rot:
         raise KernelError(f"latent_post: {rot_dims} rotated channels of {rot}")
@@ -882,7 +884,8 @@ def latent_post(proj, q_lat, cache, *, q_off: int, ckr_off: int, norm_w, eps: fl
     _gpu("positions", positions, torch.int32, (T,))
     _opt("slot_mapping", slot_mapping, torch.int32, (T,))
     _check(load("latent").tuff_latent_post(
-        proj.data_ptr(), proj.shape[1], int(q_off), int(ckr_off), q_lat.data_ptr(), cache.data_ptr(), _dt(proj),
+        proj.data_ptr(), proj.shape[1], int(q_off), int(ckr_off), q_lat.data_ptr(), cache.data_ptr(),
+        None if cache_t is None else cache_t.data_ptr(), cache.shape[2], _dt(proj),
         norm_w.data_ptr(), _dt(norm_w), float(eps), inv_freq.data_ptr() if rot_dims else None, int(rot_dims),
         positions.data_ptr(), None if slot_mapping is None else slot_mapping.data_ptr(), T, H, dim, rot, rank, _stream()),
         "latent_post")

@@ -22,8 +22,84 @@ from .base import MIXERS, Mixer, PagedKV, PositionEncoding, Runtime, WeightDecl
 from .linear import Linear
 
 
+class PagedAttention:
+    """Which attention kernels run over a paged cache, and their launch: shared by the mixers whose attention is
+    softmax(q . k * scale [- slope (i - j)]) over a request's cached positions (all of them or a window), with
+    grouped heads and optional sinks.  It reads the mixer's H, Hkv, hd, vd, window, scale, sinks, slopes."""
+
+    @staticmethod
+    def _upload(array, device):
+        """Through pinned memory, so that the host does not wait for the stream."""
+        return torch.from_numpy(array).pin_memory().to(device, non_blocking=True)
+
+    @classmethod
+    def _blocks(cls, ctx, G, nb, device, skip_single: bool = False, longest_first: bool = False):
+        key = ("query_blocks", G, nb, skip_single, longest_first)
+        blocks = ctx.host.get(key)
+        if blocks is None:
+            q_len = ctx.host["q_len"]
+            if skip_single:
+                q_len = np.where(q_len == 1, 0, q_len)
+            ctx_len = ctx.host["ctx_len"] if longest_first else None
+            blocks = ctx.host[key] = cls._upload(ops.query_blocks(q_len, G, nb, ctx_len), device)
+        return blocks
+
+    @classmethod
+    def _single_token_runs(cls, ctx, G, device):
+        """Runs of neighbouring requests with one token each in a step that also holds portions:
+        [(first token, tokens, block list, request records relative to the first token, longest
+        context)], made once a step.  Only where a request's heads fit one block of 16 columns."""
+        key = ("single_token_runs", G)
+        runs = ctx.host.get(key)
+        if runs is None:
+            runs = []
+            q_len, ctx_len = ctx.host["q_len"], ctx.host["ctx_len"]
+            if G <= 16 and (q_len == 1).any():
+                start = np.concatenate([[0], np.cumsum(q_len)[:-1]])
+                single = np.concatenate([[False], q_len == 1, [False]])
+                edges = np.flatnonzero(single[1:] != single[:-1])          # run r_lo .. r_hi - 1 for every pair
+                for r_lo, r_hi in zip(edges[0::2], edges[1::2]):
+                    tok_lo = int(start[r_lo])
+                    info = np.stack([start - tok_lo, q_len, ctx_len - q_len, ctx_len], axis=1).astype(np.int32)
+                    blocks = np.stack([np.arange(r_lo, r_hi), np.zeros(r_hi - r_lo, dtype=np.int64)], axis=1).astype(np.int32)
+                    runs.append((tok_lo, int(r_hi - r_lo), cls._upload(blocks, device), cls._upload(info, device),
+                                 int(ctx_len[r_lo:r_hi].max())))
+            ctx.host[key] = runs
+        return runs
+
+    def attend(self, q, o, ctx, cache, g) -> None:
+        G = self.H // self.Hkv
+        if self.vd == self.hd and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
+            common = dict(block_table=g.block_table, req_info=ctx.req_info, H=self.H, Hkv=self.Hkv, hd=self.hd,
+                          page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
+                          scale=self.scale, sinks=self.sinks, slopes=self.slopes)
+            if ctx.max_q_len > 1:
+                # prompt portions in the step: blocks of columns walk over their keys through LDS.
+                # Requests with a single token beside them (runs of neighbours in the step's order) go
+                # the way of a step of single tokens: one workgroup walking all keys of such a request
+                # would be the longest of the step.
+                nb = ops.attention_prefill_block_columns(self.hd) // 16
+                runs = self._single_token_runs(ctx, G, q.device)
+                # (first: with key segments it writes every row of o, the single tokens' rows come after)
+                ops.attention_prefill(q, cache.k, cache.v, o, blocks=self._blocks(ctx, G, nb, q.device, skip_single=bool(runs), longest_first=True),
+                                      positions=ctx.positions, **common)
+                for tok_lo, n, blocks, info, ctx_len in runs:
+                    ops.attention_mfma(q[tok_lo:tok_lo + n], cache.k, cache.v, o[tok_lo:tok_lo + n], blocks=blocks, nb=1,
+                                       positions=ctx.positions[tok_lo:tok_lo + n], **dict(common, req_info=info, max_ctx_len=ctx_len))
+                return
+            # single tokens: the keys of a request are split over many waves, then merged
+            nb = 1 if G <= 16 else (2 if G <= 32 or self.hd > 128 else 4)       # (wide heads: at most two column blocks a wave)
+            blocks = self._blocks(ctx, G, nb, q.device) if G > 16 * nb else None
+            ops.attention_mfma(q, cache.k, cache.v, o, blocks=blocks, nb=nb, positions=ctx.positions, **common)
+            return
+        ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
+                              req_of_token=ctx.req_of_token, positions=ctx.positions,
+                              H=self.H, Hkv=self.Hkv, hd=self.hd, page_size=cache.page_size,
+                              window=self.window or 0, scale=self.scale, vd=self.vd, sinks=self.sinks, slopes=self.slopes)
+
+
 @MIXERS.register("attention")
-class AttentionMixer(Mixer):
+class AttentionMixer(Mixer, PagedAttention):
     accepts_pending_norm = True
     adds_once_through_linear = True
 
@@ -173,73 +249,3 @@ class AttentionMixer(Mixer):
 
         ctx.run_eagerly(over_the_cache)
         self.out.forward(o, accumulate_into=residual, next_norm=next_norm)
-
-    @staticmethod
-    def _upload(array, device):
-        """Through pinned memory, so that the host does not wait for the stream."""
-        return torch.from_numpy(array).pin_memory().to(device, non_blocking=True)
-
-    @classmethod
-    def _blocks(cls, ctx, G, nb, device, skip_single: bool = False, longest_first: bool = False):
-        key = ("query_blocks", G, nb, skip_single, longest_first)
-        blocks = ctx.host.get(key)
-        if blocks is None:
-            q_len = ctx.host["q_len"]
-            if skip_single:
-                q_len = np.where(q_len == 1, 0, q_len)
-            ctx_len = ctx.host["ctx_len"] if longest_first else None
-            blocks = ctx.host[key] = cls._upload(ops.query_blocks(q_len, G, nb, ctx_len), device)
-        return blocks
-
-    @classmethod
-    def _single_token_runs(cls, ctx, G, device):
-        """Runs of neighbouring requests with one token each in a step that also holds portions:
-        [(first token, tokens, block list, request records relative to the first token, longest
-        context)], made once a step.  Only where a request's heads fit one block of 16 columns."""
-        key = ("single_token_runs", G)
-        runs = ctx.host.get(key)
-        if runs is None:
-            runs = []
-            q_len, ctx_len = ctx.host["q_len"], ctx.host["ctx_len"]
-            if G <= 16 and (q_len == 1).any():
-                start = np.concatenate([[0], np.cumsum(q_len)[:-1]])
-                single = np.concatenate([[False], q_len == 1, [False]])
-                edges = np.flatnonzero(single[1:] != single[:-1])          # run r_lo .. r_hi - 1 for every pair
-                for r_lo, r_hi in zip(edges[0::2], edges[1::2]):
-                    tok_lo = int(start[r_lo])
-                    info = np.stack([start - tok_lo, q_len, ctx_len - q_len, ctx_len], axis=1).astype(np.int32)
-                    blocks = np.stack([np.arange(r_lo, r_hi), np.zeros(r_hi - r_lo, dtype=np.int64)], axis=1).astype(np.int32)
-                    runs.append((tok_lo, int(r_hi - r_lo), cls._upload(blocks, device), cls._upload(info, device),
-                                 int(ctx_len[r_lo:r_hi].max())))
-            ctx.host[key] = runs
-        return runs
-
-    def attend(self, q, o, ctx, cache, g) -> None:
-        G = self.H // self.Hkv
-        if self.vd == self.hd and ops.attention_mfma_supported(q.dtype, self.hd, cache.page_size):
-            common = dict(block_table=g.block_table, req_info=ctx.req_info, H=self.H, Hkv=self.Hkv, hd=self.hd,
-                          page_size=cache.page_size, max_ctx_len=ctx.max_ctx_len, window=self.window or 0,
-                          scale=self.scale, sinks=self.sinks, slopes=self.slopes)
-            if ctx.max_q_len > 1:
-                # prompt portions in the step: blocks of columns walk over their keys through LDS.
-                # Requests with a single token beside them (runs of neighbours in the step's order) go
-                # the way of a step of single tokens: one workgroup walking all keys of such a request
-                # would be the longest of the step.
-                nb = ops.attention_prefill_block_columns(self.hd) // 16
-                runs = self._single_token_runs(ctx, G, q.device)
-                # (first: with key segments it writes every row of o, the single tokens' rows come after)
-                ops.attention_prefill(q, cache.k, cache.v, o, blocks=self._blocks(ctx, G, nb, q.device, skip_single=bool(runs), longest_first=True),
-                                      positions=ctx.positions, **common)
-                for tok_lo, n, blocks, info, ctx_len in runs:
-                    ops.attention_mfma(q[tok_lo:tok_lo + n], cache.k, cache.v, o[tok_lo:tok_lo + n], blocks=blocks, nb=1,
-                                       positions=ctx.positions[tok_lo:tok_lo + n], **dict(common, req_info=info, max_ctx_len=ctx_len))
-                return
-            # single tokens: the keys of a request are split over many waves, then merged
-            nb = 1 if G <= 16 else (2 if G <= 32 else 4)
-            blocks = self._blocks(ctx, G, nb, q.device) if G > 16 * nb else None
-            ops.attention_mfma(q, cache.k, cache.v, o, blocks=blocks, nb=nb, positions=ctx.positions, **common)
-            return
-        ops.attention_general(q, cache.k, cache.v, o, block_table=g.block_table,
-                              req_of_token=ctx.req_of_token, positions=ctx.positions,
-                              H=self.H, Hkv=self.Hkv, hd=self.hd, page_size=cache.page_size,
-                              window=self.window or 0, scale=self.scale, vd=self.vd, sinks=self.sinks, slopes=self.slopes)

@@ -5,7 +5,10 @@ Keys and values are expansions of one narrow row a token: with h the mixer's inp
     head a:  key = [W_uk,a c | k_r],  value = W_uv,a c,  query = [q_plain,a | rotate(q_rot,a)] from W_q h
     score = (query . key) * scale, causal softmax, head output times sigmoid((W_g h)_a) (where there is a gate), W_o.
 The cache keeps [c | k_r] and nothing else: rank + rot numbers a token, one "kv head" for all query
-heads, the row's first `rank` channels serving as the value.  The expansions are never formed for the
+heads, the row's first `rank` channels serving as the value.  Where a row is narrow enough for the
+matrix-core attention kernels (a multiple of 8, at most 256 channels) the rows are kept a second time with
+a channel's positions contiguous within the page, which is how those kernels read values; wider rows are
+kept once and go through the general kernel.  The expansions are never formed for the
 cached tokens: the query is carried into the latent space, q' = [W_uk,a^T q_plain,a | q_rot,a], attention
 runs over the cache rows as they lie, and W_uv,a is applied to the head's weighted sum of rows.
 
@@ -19,12 +22,13 @@ from typing import Optional
 import torch
 
 from ..csrc import ops
+from .attention import PagedAttention
 from .base import MIXERS, Mixer, PagedKV, Runtime, WeightDecl
 from .linear import Linear
 
 
 @MIXERS.register("latent_attention")
-class LatentAttentionMixer(Mixer):
+class LatentAttentionMixer(Mixer, PagedAttention):
     graph_safe = True
     records_portions = True
     accepts_pending_norm = True
@@ -49,6 +53,10 @@ class LatentAttentionMixer(Mixer):
             raise ValueError(f"head size {self.dk} / rank {self.rank} above {ops.HEAD_MATMUL_MAX_K}")
         self.eps, self.scale, self.rot_base = float(norm_eps), float(scale), float(rot_base)
         self.window = int(window) if window else None
+        # what PagedAttention reads: every query head against the one row a position
+        self.twice = self.lat % 8 == 0 and self.lat <= 256        # rows also kept the matrix cores' way
+        self.Hkv, self.hd, self.vd = 1, self.lat, (self.lat if self.twice else self.rank)
+        self.sinks = self.slopes = None
         self.names = dict(names)
         self.gated = "g" in self.names
         ins = [names["q"], names["dkv"]] + ([names["g"]] if self.gated else [])
@@ -64,9 +72,11 @@ class LatentAttentionMixer(Mixer):
             WeightDecl(n["uv"], (self.H * self.dv, self.rank), "normal", role="projection")]
 
     def kernel_modules(self):
-        return ["latent", "attention"]
+        return ["latent", "attention"] + (["attention_mfma", "attention_prefill"] if self.twice else [])
 
     def cache_spec(self):
+        if self.twice:
+            return PagedKV(1, self.lat, self.window)
         return PagedKV(1, self.lat, self.window, value_dim=self.rank, values_in_keys=True)
 
     def bind(self, weights, rt: Runtime):
@@ -90,7 +100,7 @@ class LatentAttentionMixer(Mixer):
         proj = self.proj.forward(h)                                           # [T, H (dk + dr) + lat + H]
         q_width = H * (dk + dr)
         q_lat = self.rt.empty(T, H * lat)
-        o_lat = self.rt.empty(T, H * rank)
+        o_lat = self.rt.empty(T, H * self.vd)         # (with the rows kept twice a head's sum is a whole row: its rotated part is not used)
         o = self.rt.empty(T, H * dv)
         # the queries' plain parts into the latent space: q'[t, a, :rank] = W_uk,a^T q_plain[t, a]
         ops.head_matmul(proj, self.w_uk, q_lat, H=H, x_head=dk + dr, y_head=lat)
@@ -99,13 +109,12 @@ class LatentAttentionMixer(Mixer):
             g = ctx.groups[cache.group]
             ops.latent_post(proj, q_lat, cache.k, q_off=0, ckr_off=q_width, norm_w=self.norm_w, eps=self.eps,
                             inv_freq=self.inv_freq, rot_dims=self.rot_dims, positions=ctx.positions,
-                            slot_mapping=g.slot_mapping if write_cache else None, H=H, dim=dk, rot=dr, rank=rank)
-            ops.attention_general(q_lat, cache.k, None, o_lat, block_table=g.block_table, req_of_token=ctx.req_of_token,
-                                  positions=ctx.positions, H=H, Hkv=1, hd=lat, vd=rank, page_size=cache.page_size,
-                                  window=self.window or 0, scale=self.scale)
+                            slot_mapping=g.slot_mapping if write_cache else None, H=H, dim=dk, rot=dr, rank=rank,
+                            cache_t=cache.v if write_cache else None)
+            self.attend(q_lat, o_lat, ctx, cache, g)
 
         ctx.run_eagerly(over_the_cache)
         # a head's value expansion of its weighted sum of latent rows, times its gate
-        ops.head_matmul(o_lat, self.w_uv, o, H=H, x_head=rank, y_head=dv,
+        ops.head_matmul(o_lat, self.w_uv, o, H=H, x_head=self.vd, y_head=dv,
                         gate=proj if self.gated else None, gate_col=q_width + lat)
         self.out.forward(o, accumulate_into=residual, next_norm=next_norm)
