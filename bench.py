@@ -358,6 +358,22 @@ def pafodra_config(size: str):
                              "norm": {"eps": 1e-5}, "layers": [kinds[i % 4] for i in range(L)]})
 
 
+def kugalorn_config(size: str):
+    """`--design kugalorn`: layers take turns between window attention (heads of 64, a window of 1,024) and latent
+    attention (heads of 64 + 32 rotated channels, a cache row of 192 + 32), every layer with experts and a shared
+    expert, over two residual streams."""
+    from tuff_amd.models.registry import config_from_dict
+    d, L, H, G, _, E, top, eff = DESIGN_SIZES[size]
+    moe = {"kind": "moe", "router": {"experts": E, "top": top}, "expert": {"ff": eff, "limit": 7.0}, "shared": {"ff": eff, "limit": 7.0}}
+    kinds = [
+        {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": 1024}}, "mlp": moe},
+        {"type": "latent_attention", "mixer": {"heads": H, "dim": 64, "rot_dim": 32, "vdim": 64, "kv_rank": 192, "scale": 0.1,
+                                               "rot": {"base": 10000.0, "dims": 32}}, "mlp": moe},
+    ]
+    return config_from_dict({"architecture": "Kugalorn", "vocab": DESIGN_VOCAB, "width": d, "norm": {"eps": 1e-6}, "streams": 2,
+                             "layers": [kinds[i % 2] for i in range(L)]})
+
+
 def lfm2_config_like(size: str):
     """The LFM2 model of the same width, depth, heads, vocabulary and dense feed-forward: its short-conv
     layers stand where the other design has its recurrences."""
@@ -436,19 +452,20 @@ def time_design(cfg, dtype: str, prefill_tokens: int, batch: int, context: int, 
 
 
 def run_design(args) -> dict:
-    """`--design pafodra`: the Pafodra decoder at sizes that resemble a real model's layers (random weights)
+    """`--design pafodra|kugalorn`: that decoder at sizes that resemble a real model's layers (random weights)
     beside the LFM2 decoder of equal width, depth and feed-forward."""
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     classes = os.environ.get("TUFF_TRACE", "")[:1] == "1"
-    out = {"design": "pafodra", "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_batch": args.batch,
+    design, make = args.design, {"pafodra": pafodra_config, "kugalorn": kugalorn_config}[args.design]
+    out = {"design": design, "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_batch": args.batch,
            "decode_context": args.design_context, "data": f"synthetic: seeded random weights (seed {SEED}), uniform random token ids",
            "sizes": {}}
     for size in args.design_sizes.split(","):
         rec = {}
-        for name, cfg in (("pafodra", pafodra_config(size)), ("lfm2", lfm2_config_like(size))):
+        for name, cfg in ((design, make(size)), ("lfm2", lfm2_config_like(size))):
             rec[name] = time_design(cfg, dtype, PREFILL_TOKENS, args.batch, args.design_context, args.point_steps, classes)
-        rec["prefill_ratio"] = round(rec["pafodra"]["prefill_tok_s"] / rec["lfm2"]["prefill_tok_s"], 3)
-        rec["decode_ratio"] = round(rec["pafodra"]["decode_tok_s"] / rec["lfm2"]["decode_tok_s"], 3)
+        rec["prefill_ratio"] = round(rec[design]["prefill_tok_s"] / rec["lfm2"]["prefill_tok_s"], 3)
+        rec["decode_ratio"] = round(rec[design]["decode_tok_s"] / rec["lfm2"]["decode_tok_s"], 3)
         out["sizes"][size] = rec
     return out
 
@@ -531,7 +548,7 @@ def main() -> int:
     ap.add_argument("--shape", default="1.2b", choices=["1.2b"] + sorted(OTHER_SHAPES),
                     help="measure another shape of the architecture in the benchmark's place (for profiling; "
                          "its points only, no other shapes after it)")
-    ap.add_argument("--design", choices=["pafodra"],
+    ap.add_argument("--design", choices=["pafodra", "kugalorn"],
                     help="instead of the benchmark: prefill and decode of another design at sizes that resemble a real "
                          "model's layers, beside the LFM2 model of equal size (TUFF_TRACE=1 adds GPU time by kernel class)")
     ap.add_argument("--design-sizes", default="1k,2k", help="with --design: which of " + ",".join(sorted(DESIGN_SIZES)))
