@@ -75,6 +75,10 @@ ONLY = {
     "attention_unmasked": config(48, 101, [layer(attn(2, 2, 24, 24, 0.4))], streams=2),
     "latent": config(48, 101, [layer(latent(2, 16, 8, 24, 32, 0.6))], streams=3),
     "latent_wide": config(64, 101, [layer(latent(3, 24, 40, 16, 280, 0.3, dims=24))], streams=2),     # a cache row of 320
+    # head counts and sizes on borders of 8 (the per-head products on the matrix cores), and a cache row of 160 with 24
+    # heads to it (wide rows, more heads than one block of columns holds)
+    "latent_eights": config(48, 101, [layer(latent(8, 16, 8, 24, 32, 0.5))], streams=2),
+    "latent_many_heads": config(64, 101, [layer(latent(24, 16, 8, 8, 152, 0.4, dims=4))], streams=1),
     "streams": config(40, 101, [layer(attn(1, 1, 8, 8, 0.3, window=4)), layer(attn(1, 1, 8, 8, 0.3, window=4))], streams=4),
     "moe": config(48, 101, [layer(attn(1, 1, 8, 8, 0.3, window=8), moe(6, 2, 24, 0.9, shared=16, shared_limit=1.4))], streams=2),
     "moe_odd": config(44, 101, [layer(attn(1, 1, 8, 8, 0.3, window=8), moe(3, 2, 20, 0.9, shared=12, shared_limit=1.4))], streams=2),

@@ -373,6 +373,37 @@ def test_latent_kernels_alone(gpu):
     assert (out.view(T, H, 5).double().cpu() - want).abs().max() < 1e-4
 
 
+@pytest.mark.parametrize("T, H, K, N, x_head, y_head, gated", [(37, 3, 40, 20, 48, 24, True), (5, 24, 16, 152, 24, 160, False),
+                                                                (130, 2, 264, 7, 272, 9, True), (16, 1, 8, 16, 8, 16, False)])
+def test_per_head_product_on_the_matrix_cores(gpu, T, H, K, N, x_head, y_head, gated):
+    """bfloat16 operands, inner sizes that are no multiples of 32, outputs that are no multiples of 16 or 4, tokens that
+    do not fill a tile, rows wider than what is read: against the float64 product of the same bfloat16 values; what lies
+    beside the written columns stays."""
+    from tuff_amd.csrc import ops
+    g = torch.Generator().manual_seed(T + K)
+    x_col, extra = 8, 8
+    x = torch.randn(T, x_col + H * x_head + extra, generator=g).to(torch.bfloat16)
+    w_nk = torch.randn(H, N, K, generator=g).to(torch.bfloat16)
+    gate = torch.randn(T, H + 3, generator=g).to(torch.bfloat16)
+    y = torch.full((T, 2 + H * y_head), 5.0, dtype=torch.bfloat16, device=gpu)
+    assert ops.head_matmul_mfma_supported(torch.bfloat16, K, x.shape[1], x_col, x_head)
+    ops.head_matmul(x.to(gpu), None, y, H=H, x_col=x_col, x_head=x_head, y_col=2, y_head=y_head, w_nk=w_nk.to(gpu),
+                    gate=gate.to(gpu) if gated else None, gate_col=3)
+    xs = x[:, x_col:x_col + H * x_head].view(T, H, x_head)[..., :K].double()
+    want = torch.einsum("thk,hnk->thn", xs, w_nk.double())
+    if gated:
+        want = want * torch.sigmoid(gate[:, 3:3 + H].double())[..., None]
+    got = y.cpu()[:, 2:].view(T, H, y_head).double()
+    err = (got[..., :N] - want).abs().max() / want.abs().max()
+    assert err < 6e-3, err                                   # one bfloat16 rounding of the result
+    assert (got[..., N:] == 5.0).all() and (y.cpu()[:, :2] == 5.0).all()
+    # the two kernels agree on a token whatever stands beside it
+    alone = torch.full((1, 2 + H * y_head), 5.0, dtype=torch.bfloat16, device=gpu)
+    ops.head_matmul(x[T - 1:].to(gpu), None, alone, H=H, x_col=x_col, x_head=x_head, y_col=2, y_head=y_head, w_nk=w_nk.to(gpu),
+                    gate=gate[T - 1:].to(gpu) if gated else None, gate_col=3)
+    assert torch.equal(alone.cpu()[0], y.cpu()[T - 1])
+
+
 # ------------------------------------------------------------------- generation, command line
 def _plain_greedy(name, prompt, n_new, seed=0):
     _, raw, w = model(name, seed)

@@ -463,7 +463,36 @@ __global__ __launch_bounds__(NW * WAVE) void attn_partition_kernel(
         }
     };
 
-    if constexpr (NW == 1) {
+    // Heads wider than 128 channels have no form of four waves to agree with, and a second set of accumulators does
+    // not fit beside the first in a wave's registers: the partition is walked as one unit.
+    constexpr bool ONE_UNIT = HDP > 128;
+    if constexpr (NW == 1 && ONE_UNIT) {
+        begin_unit();
+        for (int key0 = key_begin; key0 < key_end; key0 += UNIT) {
+            if constexpr (AHEAD) {
+                const bool more = key0 + 32 < key_end;
+                if (more) load_tile(key0 + 32, tb);
+                compute(key0, ta);
+                if (more) {
+                    if (key0 + UNIT < key_end) load_tile(key0 + UNIT, ta);
+                    compute(key0 + 32, tb);
+                }
+            } else {
+                for (int k2 = key0; k2 < min(key0 + UNIT, key_end); k2 += 32) {
+                    load_tile(k2, ta);
+                    compute(k2, ta);
+                }
+            }
+        }
+        unit_sums();
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            m_acc[nb] = m_run[nb];
+            l_acc[nb] = l_run[nb];
+#pragma unroll
+            for (int db = 0; db < DB; ++db) o_acc[db][nb] = o[db][nb];
+        }
+    } else if constexpr (NW == 1) {
         // units in ascending order, each from a fresh state, merged into the partition's result as they end
         for (int key0 = key_begin; key0 < key_end; key0 += UNIT) {
             begin_unit();

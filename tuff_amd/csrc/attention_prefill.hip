@@ -454,7 +454,7 @@ int launch(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* kc, con
 }  // namespace
 
 // Columns a block of the list must hold for this head size.
-TUFF_EXPORT int tuff_attention_prefill_block_columns(int hd) { return hd <= 128 ? 128 : 64; }
+TUFF_EXPORT int tuff_attention_prefill_block_columns(int hd) { (void)hd; return 128; }
 
 // Query blocks are listed by the host, best those with the most keys first: block b holds the columns
 // blk[b].y .. + block_columns - 1 of request blk[b].x (a request's columns are numbered (token - its first token) * G + head
@@ -490,7 +490,7 @@ TUFF_EXPORT int tuff_attention_prefill_biased(const void* q, const void* k_cache
     else if (hd <= 64) GO(64, 2, 2);
     else if (hd <= 96) GO(96, 2, 2);
     else if (hd <= 128) GO(128, 2, 2);
-    else GO(256, 1, 1);
+    else GO(256, 2, 1);
 #undef GO
 }
 

@@ -124,6 +124,57 @@ __global__ __launch_bounds__(256) void head_matmul_kernel(const T* __restrict__ 
         }
     }
 }
+
+// The same product on the matrix cores (bfloat16, K a multiple of 8 up to 32 KC, operands on 16-byte borders).  Wt is
+// [H][N][K]: a column's weights lie together, so a lane's eight k of either operand are one 16-byte load.  A workgroup
+// takes 16 tokens of one head; their x stays in registers and the four waves share the output's blocks of 16 columns.
+// The product is formed transposed (rows: output columns, columns: tokens), which leaves a lane four neighbouring
+// columns of one token.  A token's sums do not depend on the tokens beside it.
+template <int KC>
+__global__ __launch_bounds__(256) void head_matmul_mfma_kernel(const bf16_t* __restrict__ x, long long x_row, long long x_head,
+                                                               const bf16_t* __restrict__ Wt, bf16_t* __restrict__ y, long long y_row,
+                                                               long long y_head, const bf16_t* __restrict__ gate, long long gate_row,
+                                                               int n_tokens, int K, int N, int vec_store) {
+    const int h = blockIdx.y, t0 = blockIdx.x * 16;
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n16 = lane % 16, g = lane / 16;
+    const int t = t0 + n16;
+    const bool tok = t < n_tokens;
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bf16_t* xr = x + (long long)(tok ? t : 0) * x_row + h * x_head;
+    bf16x8 xf[KC];
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+        const int k = kc * 32 + g * 8;
+        xf[kc] = (tok && k < K) ? *(const bf16x8*)(xr + k) : zero;
+    }
+    float gv = 1.f;
+    if (gate && tok) gv = 1.0f / (1.0f + expf(-to_f32(gate[(long long)t * gate_row + h])));
+    const bf16_t* Wh = Wt + (long long)h * N * K;
+    for (int nb = wave; nb * 16 < N; nb += 4) {
+        const int n = nb * 16 + n16;
+        const bf16_t* wr = Wh + (long long)(n < N ? n : 0) * K;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) {
+            const int k = kc * 32 + g * 8;
+            const bf16x8 wf = (n < N && k < K) ? *(const bf16x8*)(wr + k) : zero;
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[kc], acc, 0, 0, 0);
+        }
+        if (!tok) continue;
+        const int col = nb * 16 + 4 * g;               // acc[e]: column col + e of token t
+        bf16_t* dst = y + (long long)t * y_row + h * y_head + col;
+        if (vec_store && col + 3 < N) {
+            bf16x4 o4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o4[e] = (bf16_t)(acc[e] * gv);
+            *(bf16x4*)dst = o4;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < N) dst[e] = (bf16_t)(acc[e] * gv);
+        }
+    }
+}
 }  // namespace
 
 // proj [T][row_stride] of type dt holds, a token: the heads' queries [H][dim + rot] from q_off, the latent's raw
@@ -165,5 +216,26 @@ TUFF_EXPORT int tuff_head_matmul(const void* x, long long x_row, long long x_hea
     else
         hipLaunchKernelGGL(head_matmul_kernel<bf16_t>, grid, block, lds, stream, (const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
                            (bf16_t*)y, y_row, y_head, (const bf16_t*)gate, gate_row, n_tokens, K, N);
+    return launch_status();
+}
+
+// The matrix-core form of the product above: bfloat16; Wt is the weight as [H][N][K].  K must be a multiple of 8 and at
+// most 512, and x, x_row, x_head must keep every head's row on a 16-byte border (returns -2 otherwise: the caller
+// takes the other kernel).
+TUFF_EXPORT int tuff_head_matmul_mfma(const void* x, long long x_row, long long x_head, const void* Wt, void* y, long long y_row,
+                                      long long y_head, const void* gate, long long gate_row, int n_tokens, int H, int K, int N,
+                                      hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (H < 1 || H > 65535 || K < 8 || K % 8 || K > 512 || N < 1) return -2;
+    if ((uintptr_t)x % 16 || (uintptr_t)Wt % 16 || x_row % 8 || x_head % 8) return -2;
+    const int vec_store = ((uintptr_t)y % 8 == 0 && y_row % 4 == 0 && y_head % 4 == 0) ? 1 : 0;
+    dim3 grid(ceil_div(n_tokens, 16), H), block(256);
+#define LAUNCH(KC) hipLaunchKernelGGL(head_matmul_mfma_kernel<KC>, grid, block, 0, stream, (const bf16_t*)x, x_row, x_head, \
+        (const bf16_t*)Wt, (bf16_t*)y, y_row, y_head, (const bf16_t*)gate, gate_row, n_tokens, K, N, vec_store)
+    if (K <= 64) LAUNCH(2);
+    else if (K <= 128) LAUNCH(4);
+    else if (K <= 256) LAUNCH(8);
+    else LAUNCH(16);
+#undef LAUNCH
     return launch_status();
 }

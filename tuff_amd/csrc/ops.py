@@ -106,6 +106,8 @@ _SIGNATURES = {
                              _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tuff_head_matmul": [_c_void_p, _c_ll, _c_ll, _c_void_p, _c_void_p, _c_ll, _c_ll, _c_void_p, _c_ll, _c_int,
                              _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tuff_head_matmul_mfma": [_c_void_p, _c_ll, _c_ll, _c_void_p, _c_void_p, _c_ll, _c_ll, _c_void_p, _c_ll,
+                                  _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "attention_mfma": {
         "tuff_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
@@ -894,10 +896,46 @@ def latent_post(proj, q_lat, cache, *, q_off: int, ckr_off: int, norm_w, eps: fl
 HEAD_MATMUL_MAX_K = 2048
 
 
-def head_matmul(x, w, y, *, H: int, x_col: int = 0, x_head: int, y_col: int = 0, y_head: int, gate=None, gate_col: int = 0) -> None:
+HEAD_MATMUL_MFMA_MAX_K = 512
+
+
+def head_matmul_mfma_supported(dtype, K: int, x_width: int, x_col: int, x_head: int) -> bool:
+    """Whether the matrix-core form takes these operands: bfloat16, an inner size that is a multiple of 8 up to 512,
+    every head's row of x on a 16-byte border."""
+    return (dtype == torch.bfloat16 and K % 8 == 0 and 8 <= K <= HEAD_MATMUL_MFMA_MAX_K
+            and x_width % 8 == 0 and x_col % 8 == 0 and x_head % 8 == 0)
+
+
+def head_matmul(x, w, y, *, H: int, x_col: int = 0, x_head: int, y_col: int = 0, y_head: int, gate=None, gate_col: int = 0,
+                w_nk=None) -> None:
     """y[t, y_col + h * y_head + n] = sum_k x[t, x_col + h * x_head + k] * w[h, k, n], n < N, k < K, for w [H, K, N];
     with gate ([T, *], its column gate_col + h the head's) times sigmoid(gate).  x, w, y, gate of one type; rows of x, y
-    and gate may be wider than what is read or written."""
+    and gate may be wider than what is read or written.  w_nk: the same weights as [H, N, K]; where it is given and
+    head_matmul_mfma_supported() holds the product runs on the matrix cores (w may then be None)."""
+    if w_nk is not None and head_matmul_mfma_supported(x.dtype, w_nk.shape[2], x.shape[1], x_col, x_head):
+        T = x.shape[0]
+        Hw, N, K = w_nk.shape
+        _gpu("x", x, torch.bfloat16, (T, None))
+        _gpu("w_nk", w_nk, torch.bfloat16)
+        _gpu("y", y, torch.bfloat16, (T, None))
+        if Hw != H:
+            raise KernelError(f"head_matmul: w_nk is {tuple(w_nk.shape)} for {H} heads")
+        if x_col + (H - 1) * x_head + K > x.shape[1] or y_col + (H - 1) * y_head + N > y.shape[1] or min(x_col, y_col) < 0:
+            raise KernelError("head_matmul: the heads' columns lie outside a row")
+        if x_head < 0 or (y_head < N and H > 1):
+            raise KernelError("head_matmul: the heads' outputs overlap")
+        gp = None
+        if gate is not None:
+            _gpu("gate", gate, torch.bfloat16, (T, None))
+            if gate_col < 0 or gate_col + H > gate.shape[1]:
+                raise KernelError("head_matmul: the gates' columns lie outside a row")
+            gp = gate.data_ptr() + gate_col * 2
+        _check(load("latent").tuff_head_matmul_mfma(
+            x.data_ptr() + x_col * 2, x.shape[1], int(x_head), w_nk.data_ptr(), y.data_ptr() + y_col * 2, y.shape[1], int(y_head),
+            gp, 0 if gate is None else gate.shape[1], T, H, K, N, _stream()), "head_matmul_mfma")
+        return
+    if w is None:
+        raise KernelError("head_matmul: these operands need the weights as [H, K, N]")
     T = x.shape[0]
     dt = x.dtype
     Hw, K, N = w.shape
@@ -1041,7 +1079,7 @@ def attention_decode_fused(qkv, k_cache, v_cache, out, *, block_table, req_info,
 
 def attention_prefill_block_columns(hd: int) -> int:
     """Columns (token, head in the kv group) a query block of attention_prefill holds."""
-    return 128 if hd <= 128 else 64
+    return 128
 
 
 PREFILL_WORKGROUP_SLOTS = 512    # workgroups of attention_prefill the part runs side by side (two a CU); with at most

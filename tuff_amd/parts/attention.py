@@ -88,7 +88,8 @@ class PagedAttention:
                                        positions=ctx.positions[tok_lo:tok_lo + n], **dict(common, req_info=info, max_ctx_len=ctx_len))
                 return
             # single tokens: the keys of a request are split over many waves, then merged
-            nb = 1 if G <= 16 else (2 if G <= 32 or self.hd > 128 else 4)       # (wide heads: at most two column blocks a wave)
+            # (heads wider than 128 channels: one column block a wave, which leaves registers to load a step's keys ahead)
+            nb = 1 if G <= 16 or self.hd > 128 else (2 if G <= 32 else 4)
             blocks = self._blocks(ctx, G, nb, q.device) if G > 16 * nb else None
             ops.attention_mfma(q, cache.k, cache.v, o, blocks=blocks, nb=nb, positions=ctx.positions, **common)
             return

@@ -90,6 +90,12 @@ class LatentAttentionMixer(Mixer, PagedAttention):
         # to [H][rank][vdim], so that both per-head products read a weight row a step of the inner index.
         self.w_uk = weights[n["uk"]].to(dt).reshape(self.H, self.dk, self.rank).contiguous()
         self.w_uv = weights[n["uv"]].to(dt).reshape(self.H, self.dv, self.rank).transpose(1, 2).contiguous()
+        # the matrix-core form of those products reads a column's weights together: [H][rank][dim] and [H][vdim][rank]
+        self.w_uk_nk = self.w_uv_nk = None
+        if ops.head_matmul_mfma_supported(dt, self.dk, self.proj.out_features, 0, self.dk + self.dr):
+            self.w_uk_nk = self.w_uk.transpose(1, 2).contiguous()
+        if ops.head_matmul_mfma_supported(dt, self.rank, self.H * self.vd, 0, self.vd):
+            self.w_uv_nk = weights[n["uv"]].to(dt).reshape(self.H, self.dv, self.rank).contiguous()
         half = self.rot_dims // 2
         self.inv_freq = torch.tensor([self.rot_base ** (-2.0 * i / self.rot_dims) for i in range(half)],
                                      dtype=torch.float64).to(torch.float32).to(rt.device)
@@ -103,7 +109,7 @@ class LatentAttentionMixer(Mixer, PagedAttention):
         o_lat = self.rt.empty(T, H * self.vd)         # (with the rows kept twice a head's sum is a whole row: its rotated part is not used)
         o = self.rt.empty(T, H * dv)
         # the queries' plain parts into the latent space: q'[t, a, :rank] = W_uk,a^T q_plain[t, a]
-        ops.head_matmul(proj, self.w_uk, q_lat, H=H, x_head=dk + dr, y_head=lat)
+        ops.head_matmul(proj, self.w_uk, q_lat, H=H, x_head=dk + dr, y_head=lat, w_nk=self.w_uk_nk)
 
         def over_the_cache(ctx):
             g = ctx.groups[cache.group]
@@ -116,5 +122,5 @@ class LatentAttentionMixer(Mixer, PagedAttention):
         ctx.run_eagerly(over_the_cache)
         # a head's value expansion of its weighted sum of latent rows, times its gate
         ops.head_matmul(o_lat, self.w_uv, o, H=H, x_head=self.vd, y_head=dv,
-                        gate=proj if self.gated else None, gate_col=q_width + lat)
+                        gate=proj if self.gated else None, gate_col=q_width + lat, w_nk=self.w_uv_nk)
         self.out.forward(o, accumulate_into=residual, next_norm=next_norm)
