@@ -404,6 +404,37 @@ def test_per_head_product_on_the_matrix_cores(gpu, T, H, K, N, x_head, y_head, g
     assert torch.equal(alone.cpu()[0], y.cpu()[T - 1])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d, E, top", [(44, 5, 2), (50, 3, 3), (256, 16, 2)])
+def test_router_of_a_long_step_gives_the_bits_of_a_short_one(gpu, d, E, top, dtype):
+    """A step of a thousand tokens and more takes several tokens a workgroup; a token's logits, choice and weights are
+    those it gets in a short step, bit for bit, and the float64 ones up to rounding (a count that fills no workgroup)."""
+    from tuff_amd.csrc import ops
+    g = torch.Generator().manual_seed(d)
+    T = 1027
+    h = torch.randn(T, d, generator=g).to(dtype)
+    w = torch.randn(E, d, generator=g) / d ** 0.5
+    b = torch.randn(E, generator=g)
+
+    def run(rows):
+        n = rows.shape[0]
+        z = torch.zeros(n, E, device=gpu)
+        ids = torch.zeros(n, top, dtype=torch.int32, device=gpu)
+        wts = torch.zeros(n, top, device=gpu)
+        ops.moe_router(rows.to(gpu), w.to(gpu), z, ids, wts, E=E, top=top, weights="softmax", bias=b.to(gpu))
+        return z.cpu(), ids.cpu(), wts.cpu()
+    z, ids, wts = run(h)
+    for lo, hi in ((0, 9), (1020, 1027), (511, 512)):
+        z1, ids1, wts1 = run(h[lo:hi])
+        assert torch.equal(z[lo:hi], z1) and torch.equal(ids[lo:hi], ids1) and torch.equal(wts[lo:hi], wts1)
+    want = h.double() @ w.double().T + b.double()
+    assert (z.double() - want).abs().max() < 1e-4
+    best = want.topk(top, dim=1)
+    clear = (best.values[:, -1] - want.topk(min(top + 1, E), dim=1).values[:, -1]).abs() > 1e-3 if top < E else torch.ones(T, dtype=torch.bool)
+    assert torch.equal(ids[clear].long().sort(1).values, best.indices[clear].sort(1).values)
+    assert (wts.sum(1) - 1).abs().max() < 1e-5
+
+
 # ------------------------------------------------------------------- generation, command line
 def _plain_greedy(name, prompt, n_new, seed=0):
     _, raw, w = model(name, seed)

@@ -68,40 +68,57 @@ __global__ void route_kernel(const float* __restrict__ z, int stride, int* __res
 // that are wanted as float32 products of the same rows).
 constexpr int ROUTER_WAVES = 16;
 
-template <typename T>
+// TB tokens a workgroup: a wave keeps a piece of its row of W in registers for all of them, so the row is asked for
+// once a workgroup.  A token's sums are the same chain whatever TB is.
+template <typename T, int TB>
 __global__ __launch_bounds__(ROUTER_WAVES * WAVE) void router_kernel(const T* __restrict__ h, const float* __restrict__ W,
                                                                       float* __restrict__ z, int* __restrict__ ids,
-                                                                      float* __restrict__ wts, int d, int N, int E, int top,
+                                                                      float* __restrict__ wts, int n_tokens, int d, int N, int E, int top,
                                                                       int weight_fn, const float* __restrict__ bias) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
-    float* xs = sm;                                        // d floats, padded to a multiple of 4
-    float* zs = sm + ((d + 3) & ~3);
-    const long long t = blockIdx.x;
-    for (int c = threadIdx.x; c < d; c += ROUTER_WAVES * WAVE) xs[c] = to_f32(h[t * d + c]);
+    const int dp = (d + 3) & ~3;
+    float* xs = sm;                                        // TB rows of d floats, each padded to a multiple of 4
+    float* zs = sm + TB * dp;                              // TB rows of N logits
+    const long long t0 = (long long)blockIdx.x * TB;
+    const int nt = (int)min((long long)TB, n_tokens - t0);
+    for (int b = 0; b < TB; ++b)
+        for (int c = threadIdx.x; c < d; c += ROUTER_WAVES * WAVE) xs[b * dp + c] = b < nt ? to_f32(h[(t0 + b) * d + c]) : 0.f;
     __syncthreads();
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     for (int n = wave; n < N; n += ROUTER_WAVES) {
         const float* wr = W + (long long)n * d;
-        float acc = 0.f;
+        float acc[TB];
+#pragma unroll
+        for (int b = 0; b < TB; ++b) acc[b] = 0.f;
         if (d % 4 == 0) {
             // four neighbouring terms a lane and step, several steps' loads under way at a time
 #pragma unroll 8
             for (int c = lane * 4; c < d; c += 4 * WAVE) {
                 const f32x4 w4 = *(const f32x4*)(wr + c);
-                const f32x4 x4 = *(const f32x4*)(xs + c);
-                acc = fmaf(w4[0], x4[0], acc); acc = fmaf(w4[1], x4[1], acc);
-                acc = fmaf(w4[2], x4[2], acc); acc = fmaf(w4[3], x4[3], acc);
+#pragma unroll
+                for (int b = 0; b < TB; ++b) {
+                    const f32x4 x4 = *(const f32x4*)(xs + b * dp + c);
+                    acc[b] = fmaf(w4[0], x4[0], acc[b]); acc[b] = fmaf(w4[1], x4[1], acc[b]);
+                    acc[b] = fmaf(w4[2], x4[2], acc[b]); acc[b] = fmaf(w4[3], x4[3], acc[b]);
+                }
             }
         } else {
 #pragma unroll 8
-            for (int c = lane; c < d; c += WAVE) acc = fmaf(wr[c], xs[c], acc);
+            for (int c = lane; c < d; c += WAVE) {
+                const float w = wr[c];
+#pragma unroll
+                for (int b = 0; b < TB; ++b) acc[b] = fmaf(w, xs[b * dp + c], acc[b]);
+            }
         }
-        acc = wave_sum(acc);
-        if (bias && n < E) acc += bias[n];
-        if (lane == 0) { zs[n] = acc; z[t * N + n] = acc; }
+#pragma unroll
+        for (int b = 0; b < TB; ++b) {
+            float a = wave_sum(acc[b]);
+            if (bias && n < E) a += bias[n];
+            if (lane == 0 && b < nt) { zs[b * N + n] = a; z[(t0 + b) * N + n] = a; }
+        }
     }
     __syncthreads();
-    if (threadIdx.x == 0) choose(zs, ids, wts, t, E, top, weight_fn);
+    if (threadIdx.x < nt) choose(zs + threadIdx.x * N, ids, wts, t0 + threadIdx.x, E, top, weight_fn);
 }
 
 constexpr int ROWS_WG = 16;          // output rows a workgroup of four waves computes
@@ -332,9 +349,15 @@ TUFF_EXPORT int tuff_moe_router(const void* h, int dt, const float* W, float* z,
                                 int N, int E, int top, int weight_fn, const float* bias, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (top < 1 || top > E || N < E || (long long)(d + 4 + N) * 4 > 65536) return -2;
-    const size_t lds = (size_t)(((d + 3) & ~3) + N) * sizeof(float);
-    if (dt == DT_F32) hipLaunchKernelGGL(router_kernel<float>, dim3(n_tokens), dim3(ROUTER_WAVES * WAVE), lds, stream, (const float*)h, W, z, ids, wts, d, N, E, top, weight_fn, bias);
-    else hipLaunchKernelGGL(router_kernel<bf16_t>, dim3(n_tokens), dim3(ROUTER_WAVES * WAVE), lds, stream, (const bf16_t*)h, W, z, ids, wts, d, N, E, top, weight_fn, bias);
+    // long steps: four tokens a workgroup where that fits the LDS (the rows of W are then read a quarter as often)
+    const bool four = n_tokens >= 1024 && (long long)(d + 4 + N) * 16 <= 65536;
+    const int TB = four ? 4 : 1;
+    const size_t lds = (size_t)TB * (((d + 3) & ~3) + N) * sizeof(float);
+    const dim3 grid((unsigned)ceil_div(n_tokens, TB)), block(ROUTER_WAVES * WAVE);
+#define LAUNCH(T, B) hipLaunchKernelGGL((router_kernel<T, B>), grid, block, lds, stream, (const T*)h, W, z, ids, wts, n_tokens, d, N, E, top, weight_fn, bias)
+    if (dt == DT_F32) { if (four) LAUNCH(float, 4); else LAUNCH(float, 1); }
+    else { if (four) LAUNCH(bf16_t, 4); else LAUNCH(bf16_t, 1); }
+#undef LAUNCH
     return launch_status();
 }
 
