@@ -435,6 +435,33 @@ def test_router_of_a_long_step_gives_the_bits_of_a_short_one(gpu, d, E, top, dty
     assert (wts.sum(1) - 1).abs().max() < 1e-5
 
 
+def test_experts_in_tall_tiles_give_the_same_bits(gpu):
+    """Steps with many rows an expert and wide matrices take tiles of 64 rows; a row's result does not depend on the
+    tile it is in.  The width from which that form is taken is lowered for the test."""
+    from tuff_amd.csrc import ops
+    lib = ops.load("moe")
+    g = torch.Generator().manual_seed(3)
+    T, d, F, E, top = 170, 64, 40, 2, 2
+    h = torch.randn(T, d, generator=g).to(torch.bfloat16).to(gpu)
+    mats = lambda n, k: [(torch.randn(n, k, generator=g) * k ** -0.5).to(torch.bfloat16) for _ in range(E)]
+    up_t = ops.tile_experts([ops.interleave_gate_up(a, b) for a, b in zip(mats(F, d), mats(F, d))]).to(gpu)
+    down_t = ops.tile_experts(mats(d, F)).to(gpu)
+    ids = torch.tensor([[0, 1]] * T, dtype=torch.int32, device=gpu)
+    wts = torch.rand(T, top, generator=g).to(gpu)
+    got = []
+    old = lib.tuff_moe_grouped_wide_from(-1)
+    try:
+        for wide in (1 << 30, 0):
+            lib.tuff_moe_grouped_wide_from(wide)
+            res = torch.zeros(T, d, device=gpu)
+            ops.moe_experts_grouped(h, up_t, down_t, ids, wts, res, F=F, activation="swish_clamp", scale_input=False, gated=True,
+                                    limit=0.8, alpha=1.702)
+            got.append(res.cpu())
+    finally:
+        lib.tuff_moe_grouped_wide_from(old)
+    assert got[0].abs().max() > 0 and torch.equal(got[0], got[1])
+
+
 # ------------------------------------------------------------------- generation, command line
 def _plain_greedy(name, prompt, n_new, seed=0):
     _, raw, w = model(name, seed)
