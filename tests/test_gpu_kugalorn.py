@@ -113,6 +113,7 @@ def test_each_mechanism_alone(gpu, name, dtype):
     reqs = requests(name, [37, 1, 9])
     check(name, dtype, util.plan_whole(reqs), reqs)
     check(name, dtype, util.plan_chunks(reqs, sizes=(2, 5, 1, 3, 16, 2)), reqs)
+    check(name, dtype, util.plan_tail(reqs, tail=20), reqs)
 
 
 # -------------------------------------------------------------- whole models under every plan
