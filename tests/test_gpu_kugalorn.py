@@ -436,31 +436,42 @@ def test_router_of_a_long_step_gives_the_bits_of_a_short_one(gpu, d, E, top, dty
     assert (wts.sum(1) - 1).abs().max() < 1e-5
 
 
-def test_experts_in_tall_tiles_give_the_same_bits(gpu):
-    """Steps with many rows an expert and wide matrices take tiles of 64 rows; a row's result does not depend on the
-    tile it is in.  The width from which that form is taken is lowered for the test."""
+@pytest.mark.parametrize("T, d, F, E, top, gated, on_input", [(170, 64, 40, 2, 2, True, False), (300, 72, 136, 5, 2, True, False),
+                                                            (260, 200, 24, 3, 1, False, False), (129, 128, 128, 1, 1, True, False),
+                                                            (200, 96, 264, 4, 3, False, True)])
+def test_experts_in_other_tiles_give_the_same_bits(gpu, T, d, F, E, top, gated, on_input):
+    """Steps with many rows an expert take block tiles of 128 rows through LDS, or (wide matrices) tiles of 64 rows; a
+    row's result does not depend on the tile it is in or the kernel that formed it: inner sizes that are no multiples
+    of 64, widths that are no multiples of 128, tiles that are not full, an expert nobody chose, the choice's weight on the experts' inputs.  The row counts and
+    widths from which those forms are taken are lowered for the test."""
     from tuff_amd.csrc import ops
     lib = ops.load("moe")
-    g = torch.Generator().manual_seed(3)
-    T, d, F, E, top = 170, 64, 40, 2, 2
+    g = torch.Generator().manual_seed(T + d)
     h = torch.randn(T, d, generator=g).to(torch.bfloat16).to(gpu)
     mats = lambda n, k: [(torch.randn(n, k, generator=g) * k ** -0.5).to(torch.bfloat16) for _ in range(E)]
-    up_t = ops.tile_experts([ops.interleave_gate_up(a, b) for a, b in zip(mats(F, d), mats(F, d))]).to(gpu)
-    down_t = ops.tile_experts(mats(d, F)).to(gpu)
-    ids = torch.tensor([[0, 1]] * T, dtype=torch.int32, device=gpu)
+    first = [ops.interleave_gate_up(a, b) for a, b in zip(mats(F, d), mats(F, d))] if gated else mats(F, d)
+    up_t, down_t = ops.tile_experts(first).to(gpu), ops.tile_experts(mats(d, F)).to(gpu)
+    ids = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)])
+    if E > 2:
+        ids[ids == E - 1] = 0 if top == 1 else E - 1          # (with one choice a token: nobody takes the last expert)
+    ids = ids.to(torch.int32).to(gpu)
     wts = torch.rand(T, top, generator=g).to(gpu)
+    form = dict(F=F, scale_input=on_input, gated=gated,
+                **(dict(activation="swish_clamp", limit=0.8, alpha=1.702) if gated else dict(activation="relu2" if on_input else "gelu_tanh")))
     got = []
-    old = lib.tuff_moe_grouped_wide_from(-1)
+    old = lib.tuff_moe_grouped_wide_from(-1), lib.tuff_moe_grouped_tiled_from(-1)
     try:
-        for wide in (1 << 30, 0):
+        for wide, tiled in ((1 << 30, 1 << 30), (0, 1 << 30), (1 << 30, 0)):
             lib.tuff_moe_grouped_wide_from(wide)
+            lib.tuff_moe_grouped_tiled_from(tiled)
             res = torch.zeros(T, d, device=gpu)
-            ops.moe_experts_grouped(h, up_t, down_t, ids, wts, res, F=F, activation="swish_clamp", scale_input=False, gated=True,
-                                    limit=0.8, alpha=1.702)
+            ops.moe_experts_grouped(h, up_t, down_t, ids, wts, res, **form)
             got.append(res.cpu())
     finally:
-        lib.tuff_moe_grouped_wide_from(old)
-    assert got[0].abs().max() > 0 and torch.equal(got[0], got[1])
+        lib.tuff_moe_grouped_wide_from(old[0])
+        lib.tuff_moe_grouped_tiled_from(old[1])
+    assert got[0].abs().max() > 0 and torch.isfinite(got[0]).all()
+    assert torch.equal(got[0], got[1]) and torch.equal(got[0], got[2])
 
 
 # ------------------------------------------------------------------- generation, command line

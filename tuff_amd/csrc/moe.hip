@@ -361,11 +361,162 @@ TUFF_EXPORT int tuff_moe_router(const void* h, int dt, const float* W, float* z,
     return launch_status();
 }
 
+// The experts of steps with many rows an expert: block tiles of 128 rows of one expert x 128 rows of its matrix, the
+// operands of a step of 64 k staged through LDS and shared by the workgroup's eight waves (2 x 4, each 64 rows x 32
+// features as 4 x 2 products), so an expert's matrix is read once for 128 rows where grouped_kernel reads it once for
+// 32.  Two LDS buffers: while a step is multiplied out of one, the next step's operands travel from memory into
+// registers and then into the other; one barrier a step.  X rows lie in LDS row-major with their 16-byte chunks
+// exchanged (chunk c of row r at position c ^ (r % 8)), W as in memory (1 KB blocks, lane l's operand at 16 l).
+// The products of a row run over k in ascending steps of 32 with one accumulator, as in grouped_kernel: the two
+// kernels give the same bits, and a row's result does not depend on its tile.
+constexpr int GT_BM = 128, GT_BN = 128, GT_BK = 64, GT_NT = 512;
+
+__device__ __forceinline__ int gt_swz(int r, int c) { return r * GT_BK + ((c ^ (r % 8)) * 8); }
+
+template <bool UP>
+__global__ __launch_bounds__(GT_NT) void grouped_tiled_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                              const int* __restrict__ tiles, const int* __restrict__ sorted,
+                                                              const float* __restrict__ wts, bf16_t* __restrict__ A,
+                                                              float* __restrict__ Y, int K, int N, int top, int act, int scale_input,
+                                                              int gated, float limit, float alpha) {
+    extern __shared__ __attribute__((aligned(16))) bf16_t gt_lds[];     // [2][BM * BK] of X, then [2][BN * BK] of W
+    const int tile = blockIdx.x;
+    const int e = tiles[3 * tile];
+    if (e < 0) return;
+    const int pos0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+    const int n0 = blockIdx.y * GT_BN;
+    const int NT16 = (N + 15) / 16, KB = (K + 31) / 32;
+    bf16_t* As = gt_lds;
+    bf16_t* Bs = gt_lds + 2 * GT_BM * GT_BK;
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE, r16 = lane % 16, g = lane / 16;
+    const int wm = (wave / 4) * 64, wn = (wave % 4) * 32;
+
+    // what this thread moves a step: two 16-byte pieces of X (rows tid / 8 and 64 further, chunk tid % 8) and two of
+    // W (piece tid % 64 of block (tid / 64) % 2 ... of row tiles tid / 128 and 4 further).  Rows beyond the tile's
+    // read its first row, row tiles beyond the matrix its last: their results are never stored.
+    const int c0 = tid % 8;
+    const bf16_t* xsrc[2];
+    int xdst[2];
+    float xscale[2];                                           // UP with scale_input: the choice's weight on the row's input
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int r = tid / 8 + p * 64;
+        const int rr = r < rows ? r : 0;
+        const long long row = UP ? sorted[pos0 + rr] / top : pos0 + rr;
+        xscale[p] = (UP && scale_input) ? wts[sorted[pos0 + rr]] : 1.f;
+        xsrc[p] = X + row * K + c0 * 8;
+        xdst[p] = gt_swz(r, c0);
+    }
+    const int wpiece = tid % 64, wh = (tid / 64) % 2;
+    const bf16_t* We = W + (long long)e * NT16 * KB * 512;
+    const bf16_t* wsrc[2];
+    int wdst[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int t = tid / 128 + p * 4;                       // row tile of the block, 0 .. 7
+        const int tt = min(n0 / 16 + t, NT16 - 1);
+        wsrc[p] = We + ((long long)tt * KB + wh) * 512 + wpiece * 8;
+        wdst[p] = (t * 2 + wh) * 512 + wpiece * 8;
+    }
+    const bf16x8_ zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8_ rx[2], rw[2];
+    auto load = [&](int kt) {
+        const int k0 = kt * GT_BK;
+        const bool in_x = k0 + c0 * 8 < K, in_w = k0 / 32 + wh < KB;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            rx[p] = in_x ? *(const bf16x8_*)(xsrc[p] + k0) : zero;
+            if (UP && scale_input) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) rx[p][i] = (bf16_t)((float)rx[p][i] * xscale[p]);
+            }
+            rw[p] = in_w ? *(const bf16x8_*)(wsrc[p] + (long long)(k0 / 32) * 512) : zero;
+        }
+    };
+    auto store = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            *(bf16x8_*)(As + buf * GT_BM * GT_BK + xdst[p]) = rx[p];
+            *(bf16x8_*)(Bs + buf * GT_BN * GT_BK + wdst[p]) = rw[p];
+        }
+    };
+    f32x4 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int nk = (K + GT_BK - 1) / GT_BK;
+    load(0);
+    store(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) load(kt + 1);
+        const bf16_t* Ab = As + buf * GT_BM * GT_BK;
+        const bf16_t* Bb = Bs + buf * GT_BN * GT_BK;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            bf16x8_ b[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = *(const bf16x8_*)(Bb + ((wn / 16 + j) * 2 + half) * 512 + lane * 8);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bf16x8_ a = *(const bf16x8_*)(Ab + gt_swz(wm + i * 16 + r16, half * 4 + g));
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = mfma16(b[j], a, acc[i][j]);
+            }
+        }
+        if (kt + 1 < nk) store(buf ^ 1);
+        __syncthreads();
+    }
+
+    // acc[i][j][q]: row wm + 16 i + r16 of the tile, column n0 + wn + 16 j + 4 g + q
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = wm + i * 16 + r16;
+        if (r >= rows) continue;
+        const long long own = UP ? 0 : sorted[pos0 + r];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wn + j * 16 + 4 * g;
+            if (col >= N) continue;
+            const f32x4 v = acc[i][j];
+            if (UP && gated) {
+                // rows 2f and 2f + 1 of the first matrix are feature f's gate and up
+#pragma unroll
+                for (int q = 0; q < 4; q += 2)
+                    if (col + q + 1 < N)
+                        A[(long long)(pos0 + r) * (N / 2) + (col + q) / 2] = (bf16_t)glu_fn(v[q], v[q + 1], act, limit, alpha);
+            } else if (UP) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (col + q < N) A[(long long)(pos0 + r) * N + col + q] = (bf16_t)act_fn(v[q], act);
+            } else if (col + 3 < N && N % 4 == 0) {
+                *(f32x4*)(Y + own * N + col) = v;
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (col + q < N) Y[own * N + col + q] = v[q];
+            }
+        }
+    }
+}
+
 // From which width of both matrices on (rows of the first, rows of the second) steps with many rows an expert take
 // tiles of 64 rows.  Measured, 2,048 tokens with gated experts: hidden size 4,096, 32 experts of 1,536, four chosen:
 // 1.25 ms against 1.62 ms with tiles of 32; hidden size 2,048, 16 experts of 1,024, two chosen: 0.33 against 0.31.
 // For measurements and tests; the result does not depend on it.  Returns the value before.
 static int wide_from = 4096;
+// From how many rows an expert (on average over the step) on the experts run in block tiles of 128 rows through LDS.
+// For measurements and tests; the result does not depend on it.  Returns the value before.
+static int tiled_from = 96;
+TUFF_EXPORT int tuff_moe_grouped_tiled_from(int n) {
+    const int old = tiled_from;
+    if (n >= 0) tiled_from = n;
+    return old;
+}
+
 TUFF_EXPORT int tuff_moe_grouped_wide_from(int n) {
     const int old = wide_from;
     if (n >= 0) wide_from = n;
@@ -393,9 +544,29 @@ TUFF_EXPORT int tuff_moe_experts_grouped(const void* h, const void* w_up, const 
     // Many rows an expert and matrices wide enough to fill the chip with fewer, taller tiles: 64 rows a tile, so an
     // expert's matrix is read half as often (the caller's tile array, sized for 32 rows, is more than enough).
     if (TM == 32 && R >= 128ll * E && F1 >= wide_from && d >= wide_from) TM = 64;
-    hipLaunchKernelGGL(group_rows_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)R, E, TM, sorted, tiles, max_tiles);
     const bf16_t* H_ = (const bf16_t*)h;
     bf16_t* A_ = (bf16_t*)a;
+    // Many rows an expert: block tiles of 128 rows through LDS (the caller's tile array is sized for smaller tiles and
+    // holds these).
+    if (R >= (long long)tiled_from * E) {
+        constexpr int lds = 2 * (GT_BM + GT_BN) * GT_BK * 2;
+        static bool set = false;
+        if (!set) {
+            if (hipFuncSetAttribute((const void*)grouped_tiled_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess ||
+                hipFuncSetAttribute((const void*)grouped_tiled_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+                return -1;
+            set = true;
+        }
+        hipLaunchKernelGGL(group_rows_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)R, E, GT_BM, sorted, tiles, max_tiles);
+        hipLaunchKernelGGL(grouped_tiled_kernel<true>, dim3(max_tiles, ceil_div(F1, GT_BN)), dim3(GT_NT), lds, stream,
+                           H_, (const bf16_t*)w_up, tiles, sorted, wts, A_, nullptr, d, F1, top, act, scale_input, gated, limit, alpha);
+        hipLaunchKernelGGL(grouped_tiled_kernel<false>, dim3(max_tiles, ceil_div(d, GT_BN)), dim3(GT_NT), lds, stream,
+                           A_, (const bf16_t*)w_down, tiles, sorted, wts, nullptr, y, F, d, top, act, 0, 0, 0.f, 0.f);
+        const long long n = (long long)n_tokens * d;
+        hipLaunchKernelGGL(combine_kernel, dim3((unsigned)ceil_div_ll(n, 256)), dim3(256), 0, stream, y, wts, residual, n, d, top, !scale_input);
+        return launch_status();
+    }
+    hipLaunchKernelGGL(group_rows_kernel, dim3(1), dim3(1024), 0, stream, ids, (int)R, E, TM, sorted, tiles, max_tiles);
     // few rows an expert: many narrow workgroups stream the weights; many: wide ones reuse them
     if (TM == 64) {
         hipLaunchKernelGGL((grouped_kernel<4, 4, true>), dim3(max_tiles, ceil_div(ceil_div(F1, 16), 16)), dim3(256), 0, stream,

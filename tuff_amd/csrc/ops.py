@@ -60,6 +60,7 @@ _SIGNATURES = {
                             _c_int, _c_void_p, _c_void_p],
         "tuff_moe_grouped_tile_rows": [_c_ll, _c_int],
         "tuff_moe_grouped_wide_from": [_c_int],
+        "tuff_moe_grouped_tiled_from": [_c_int],
         "tuff_moe_experts_grouped": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                                      _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
         "tuff_moe_experts": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
