@@ -283,9 +283,12 @@ def test_streams_kernel_alone(gpu, S, d):
     x2, uo = dev(xs), torch.empty(T, d, device=gpu)
     ops.hc_step(x2, in_w=dev(in_w), u_out=uo)                                 # a read alone leaves the streams as they are
     assert torch.equal(x2.cpu(), xs) and (uo.double().cpu() - torch.einsum("s,std->td", in_w.double(), xs.double())).abs().max() < 1e-4
-    x3 = dev(xs)
-    ops.hc_step(x3, y=dev(y), mix=dev(mix), out_w=dev(out_w))                 # a write alone
-    assert (x3.double().cpu() - new).abs().max() < 1e-4
+    x3, y3 = dev(xs), dev(y)
+    ops.hc_step(x3, y=y3, mix=dev(mix), out_w=dev(out_w))                     # a write alone
+    assert (x3.double().cpu() - new).abs().max() < 1e-4 and torch.equal(y3.cpu(), y)
+    x4, y4 = dev(xs), dev(y)
+    ops.hc_step(x4, y=y4, mix=dev(mix), out_w=dev(out_w), clear_y=True)       # the sublayer's output is left cleared
+    assert torch.equal(x4, x3) and not y4.any()
 
 
 @pytest.mark.parametrize("d, F, E, top", [(64, 40, 4, 2), (44, 20, 3, 3), (128, 256, 16, 1)])

@@ -14,11 +14,11 @@ namespace {
 constexpr int MAX_STREAMS = 8;
 
 template <typename TO>
-__global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ xs, const float* __restrict__ y,
+__global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ xs, float* __restrict__ y,
                                                       const float* __restrict__ mix, const float* __restrict__ out_w,
                                                       const float* __restrict__ in_w, const float* __restrict__ norm_w,
                                                       TO* __restrict__ h_out, float* __restrict__ u_out,
-                                                      int S, long long T, int d, float eps) {
+                                                      int S, long long T, int d, float eps, int clear_y) {
     extern __shared__ float us[];                      // d floats: the row of u
     __shared__ float scratch[4];
     __shared__ float w_mix[MAX_STREAMS * MAX_STREAMS], w_out[MAX_STREAMS], w_in[MAX_STREAMS];
@@ -39,6 +39,7 @@ __global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ xs, co
         for (int s = 0; s < MAX_STREAMS; ++s) x[s] = s < S ? xs[s * plane + at] : 0.f;
         if (write) {
             const float yv = y[at];
+            if (clear_y) y[at] = 0.f;              // the sublayers add into y: it is left ready for the next one
             float nx[MAX_STREAMS];
 #pragma unroll
             for (int r = 0; r < MAX_STREAMS; ++r) {
@@ -72,10 +73,10 @@ __global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ xs, co
 
 // xs float32 [S][T][d].  mix [S][S] and out_w [S] with y [T][d]: the write (all three null: none).  in_w [S]: the
 // read (null: none); with norm_w [d] the result norm(u) * norm_w goes to h_out [T][d] of type out_dt, without it
-// u goes to u_out [T][d] in float32.
-TUFF_EXPORT int tuff_hc_step(float* xs, const float* y, const float* mix, const float* out_w, const float* in_w,
+// u goes to u_out [T][d] in float32.  clear_y: y is zero afterwards.
+TUFF_EXPORT int tuff_hc_step(float* xs, float* y, const float* mix, const float* out_w, const float* in_w,
                              const float* norm_w, void* h_out, int out_dt, float* u_out, int S, int n_tokens, int d,
-                             float eps, hipStream_t stream) {
+                             float eps, int clear_y, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (S < 1 || S > MAX_STREAMS || d < 1 || d > 15360) return -2;
     if ((mix == nullptr) != (out_w == nullptr) || (mix == nullptr) != (y == nullptr)) return -2;
@@ -83,9 +84,9 @@ TUFF_EXPORT int tuff_hc_step(float* xs, const float* y, const float* mix, const 
     const size_t lds = (size_t)d * sizeof(float);
     if (out_dt == DT_F32)
         hipLaunchKernelGGL(hc_step_kernel<float>, dim3(n_tokens), dim3(256), lds, stream, xs, y, mix, out_w, in_w, norm_w,
-                           (float*)h_out, u_out, S, (long long)n_tokens, d, eps);
+                           (float*)h_out, u_out, S, (long long)n_tokens, d, eps, clear_y);
     else
         hipLaunchKernelGGL(hc_step_kernel<bf16_t>, dim3(n_tokens), dim3(256), lds, stream, xs, y, mix, out_w, in_w, norm_w,
-                           (bf16_t*)h_out, u_out, S, (long long)n_tokens, d, eps);
+                           (bf16_t*)h_out, u_out, S, (long long)n_tokens, d, eps, clear_y);
     return launch_status();
 }

@@ -101,7 +101,7 @@ _SIGNATURES = {
     },
     "hyper": {
         "tuff_hc_step": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
-                         _c_int, _c_int, _c_int, _c_float, _c_void_p],
+                         _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     },
     "latent": {
         "tuff_latent_post": [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_float,
@@ -834,11 +834,12 @@ ATTN_GENERAL_MAX_DIM = 640   # widest key or value row of the general attention 
 HC_MAX_STREAMS, HC_MAX_DIM = 8, 15360
 
 
-def hc_step(xs, *, y=None, mix=None, out_w=None, in_w=None, norm_w=None, eps: float = 0.0, h_out=None, u_out=None) -> None:
+def hc_step(xs, *, y=None, mix=None, out_w=None, in_w=None, norm_w=None, eps: float = 0.0, h_out=None, u_out=None,
+            clear_y: bool = False) -> None:
     """One kernel over the residual streams xs (float32 [S, T, d], in place).  With y [T, d], mix [S, S] (indexed
     [from, to]) and out_w [S]: xs[r] <- sum_s mix[s, r] xs[s] + out_w[r] y.  Then, with in_w [S]: u = sum_s in_w[s]
     xs[s] (of the new values); with norm_w (float32 [d]) h_out [T, d] = u / sqrt(mean(u^2) + eps) * norm_w in h_out's
-    type, without it u_out [T, d] = u in float32."""
+    type, without it u_out [T, d] = u in float32.  clear_y: y is zero afterwards (ready for the next sublayer to add into)."""
     S, T, d = xs.shape
     _gpu("xs", xs, torch.float32)
     if S > HC_MAX_STREAMS or d > HC_MAX_DIM:
@@ -857,7 +858,7 @@ def hc_step(xs, *, y=None, mix=None, out_w=None, in_w=None, norm_w=None, eps: fl
             _gpu("u_out", u_out, torch.float32, (T, d))
     p = lambda t: None if t is None else t.data_ptr()
     _check(load("hyper").tuff_hc_step(xs.data_ptr(), p(y), p(mix), p(out_w), p(in_w), p(norm_w), p(h_out),
-                                      DT_F32 if h_out is None else _dt(h_out), p(u_out), S, T, d, float(eps), _stream()), "hc_step")
+                                      DT_F32 if h_out is None else _dt(h_out), p(u_out), S, T, d, float(eps), int(bool(clear_y)), _stream()), "hc_step")
 
 
 # ------------------------------------------------------------------- latent attention

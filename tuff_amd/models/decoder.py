@@ -205,10 +205,13 @@ class DecoderModel:
             ops.embed_rows(self.embedding, ctx.tokens, xs[s], self.embedding_scale)
         carry = None
         last = len(self.schedule) - 1
+        # what the sublayers add their outputs into: cleared once here, and by the streams' kernel whenever it has read it
+        y = torch.empty(ctx.T, self.hidden_size, dtype=torch.float32, device=self.rt.device)
+        ops.fill_u32(y, 0)
         for i, run in enumerate(self.schedule):
             block = self.blocks[run.block]
             nxt = self.blocks[self.schedule[i + 1].block].first_read() if i < last else (self._ones, None, 0.0)
-            carry = block.forward(xs, ctx, self._views_of(i, cache_views), run.writes, carry=carry, next_read=nxt)
+            carry = block.forward(xs, ctx, self._views_of(i, cache_views), run.writes, carry=carry, next_read=nxt, y=y)
             if self.on_layer is not None:
                 self.on_layer(i, xs)
         if last < 0:

@@ -201,11 +201,12 @@ class HyperConnectionBlock(Block):
         """(in [S], norm weight float32 [d], eps): what the block before needs to prepare this block's first input."""
         return self.hc["1"][0], self.norm1.weight_f32, self.norm1.eps
 
-    def forward(self, xs, ctx, cache, write_cache: bool = True, carry=None, next_read=None):
+    def forward(self, xs, ctx, cache, write_cache: bool = True, carry=None, next_read=None, y=None):
         """xs float32 [S, T, d], in place.  carry: norm1(u) of this block's first sublayer where the block before
         left it (None: computed here).  next_read: (in, norm weight or None, eps) of whoever reads the streams
         next; the result of that read is returned (the normed rows in the compute type, or, without a norm weight,
-        the plain weighted sum in float32); None: nothing is read."""
+        the plain weighted sum in float32); None: nothing is read.  y: float32 [T, d] of zeros that the sublayers add
+        into (the kernel that mixes it into the streams leaves it zero again); None: made here."""
         S, T, d = xs.shape
         if S != self.S:
             raise ValueError(f"{S} streams handed to a block of {self.S}")
@@ -213,8 +214,9 @@ class HyperConnectionBlock(Block):
             carry = self.rt.empty(T, d)
             in1, w1, eps1 = self.first_read()
             ops.hc_step(xs, in_w=in1, norm_w=w1, eps=eps1, h_out=carry)
-        y = torch.empty(T, d, dtype=torch.float32, device=xs.device)
-        ops.fill_u32(y, 0)
+        if y is None:
+            y = torch.empty(T, d, dtype=torch.float32, device=xs.device)
+            ops.fill_u32(y, 0)
         kw = {"next_norm": None} if self.mixer.adds_once_through_linear else {}
         self.mixer.forward(carry, ctx, cache, y, write_cache, **kw)
         _, mix1, out1 = self.hc["1"]
@@ -222,7 +224,6 @@ class HyperConnectionBlock(Block):
             return self._write_and_read(xs, y, mix1, out1, next_read)
         in2, mix2, out2 = self.hc["2"]
         h = self._write_and_read(xs, y, mix1, out1, (in2, self.norm2.weight_f32, self.norm2.eps))
-        ops.fill_u32(y, 0)
         kw = {"next_norm": None} if self.ffn.adds_once_through_linear else {}
         self.ffn.forward(h, ctx, y, **kw)
         return self._write_and_read(xs, y, mix2, out2, next_read)
@@ -230,13 +231,13 @@ class HyperConnectionBlock(Block):
     def _write_and_read(self, xs, y, mix, out_w, read):
         T, d = y.shape
         if read is None:
-            ops.hc_step(xs, y=y, mix=mix, out_w=out_w)
+            ops.hc_step(xs, y=y, mix=mix, out_w=out_w, clear_y=True)
             return None
         in_w, norm_w, eps = read
         if norm_w is None:
             u = torch.empty(T, d, dtype=torch.float32, device=xs.device)
-            ops.hc_step(xs, y=y, mix=mix, out_w=out_w, in_w=in_w, u_out=u)
+            ops.hc_step(xs, y=y, mix=mix, out_w=out_w, in_w=in_w, u_out=u, clear_y=True)
             return u
         h = self.rt.empty(T, d)
-        ops.hc_step(xs, y=y, mix=mix, out_w=out_w, in_w=in_w, norm_w=norm_w, eps=eps, h_out=h)
+        ops.hc_step(xs, y=y, mix=mix, out_w=out_w, in_w=in_w, norm_w=norm_w, eps=eps, h_out=h, clear_y=True)
         return h
