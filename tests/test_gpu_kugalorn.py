@@ -264,7 +264,7 @@ def test_window_attention_one_key_stands_out(gpu, dk, dv, H, G, window, dtype):
 
 
 # ----------------------------------------------------------------------- kernels alone
-@pytest.mark.parametrize("S, d", [(1, 24), (3, 200), (8, 52), (2, 1024)])
+@pytest.mark.parametrize("S, d", [(1, 24), (3, 200), (8, 52), (2, 1024), (2, 50), (3, 7), (4, 2052)])
 def test_streams_kernel_alone(gpu, S, d):
     from tuff_amd.csrc import ops
     g = torch.Generator().manual_seed(S * d)

@@ -13,15 +13,17 @@
 namespace {
 constexpr int MAX_STREAMS = 8;
 
-template <typename TO>
+// V: neighbouring columns a thread takes at a time (4 where d is a multiple of 4: 16-byte loads and stores; else 1).
+template <typename TO, int V>
 __global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ xs, float* __restrict__ y,
                                                       const float* __restrict__ mix, const float* __restrict__ out_w,
                                                       const float* __restrict__ in_w, const float* __restrict__ norm_w,
                                                       TO* __restrict__ h_out, float* __restrict__ u_out,
                                                       int S, long long T, int d, float eps, int clear_y) {
-    extern __shared__ float us[];                      // d floats: the row of u
+    extern __shared__ __attribute__((aligned(16))) float us[];     // d floats: the row of u
     __shared__ float scratch[4];
     __shared__ float w_mix[MAX_STREAMS * MAX_STREAMS], w_out[MAX_STREAMS], w_in[MAX_STREAMS];
+    typedef float vec __attribute__((ext_vector_type(V)));
     const long long t = blockIdx.x;
     const bool write = mix != nullptr, read = in_w != nullptr;
     if (threadIdx.x < S * S && write) w_mix[threadIdx.x] = mix[threadIdx.x];
@@ -32,42 +34,69 @@ __global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ xs, fl
     __syncthreads();
     const long long plane = T * (long long)d;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < d; c += 256) {
+    for (int c = threadIdx.x * V; c < d; c += 256 * V) {
         const long long at = t * d + c;
-        float x[MAX_STREAMS];
+        float x[MAX_STREAMS][V];
 #pragma unroll
-        for (int s = 0; s < MAX_STREAMS; ++s) x[s] = s < S ? xs[s * plane + at] : 0.f;
+        for (int s = 0; s < MAX_STREAMS; ++s) {
+            vec v = {};
+            if (s < S) v = *(const vec*)(xs + s * plane + at);
+#pragma unroll
+            for (int e = 0; e < V; ++e) x[s][e] = v[e];
+        }
         if (write) {
-            const float yv = y[at];
-            if (clear_y) y[at] = 0.f;              // the sublayers add into y: it is left ready for the next one
-            float nx[MAX_STREAMS];
+            const vec yv = *(const vec*)(y + at);
+            if (clear_y) { const vec z = {}; *(vec*)(y + at) = z; }    // the sublayers add into y: it is left ready for the next one
 #pragma unroll
-            for (int r = 0; r < MAX_STREAMS; ++r) {
-                float a = 0.f;
+            for (int e = 0; e < V; ++e) {
+                float nx[MAX_STREAMS];
 #pragma unroll
-                for (int s = 0; s < MAX_STREAMS; ++s)
-                    if (s < S && r < S) a = fmaf(w_mix[s * S + r], x[s], a);
-                nx[r] = r < S ? fmaf(w_out[r], yv, a) : 0.f;
+                for (int r = 0; r < MAX_STREAMS; ++r) {
+                    float a = 0.f;
+#pragma unroll
+                    for (int s = 0; s < MAX_STREAMS; ++s)
+                        if (s < S && r < S) a = fmaf(w_mix[s * S + r], x[s][e], a);
+                    nx[r] = r < S ? fmaf(w_out[r], yv[e], a) : 0.f;
+                }
+#pragma unroll
+                for (int r = 0; r < MAX_STREAMS; ++r) x[r][e] = nx[r];
             }
 #pragma unroll
             for (int r = 0; r < MAX_STREAMS; ++r) {
-                x[r] = nx[r];
-                if (r < S) xs[r * plane + at] = nx[r];
+                if (r < S) {
+                    vec v;
+#pragma unroll
+                    for (int e = 0; e < V; ++e) v[e] = x[r][e];
+                    *(vec*)(xs + r * plane + at) = v;
+                }
             }
         }
         if (read) {
-            float u = 0.f;
+            vec u;
 #pragma unroll
-            for (int s = 0; s < MAX_STREAMS; ++s)
-                if (s < S) u = fmaf(w_in[s], x[s], u);
-            if (norm_w) { us[c] = u; ss = fmaf(u, u, ss); }
-            else u_out[at] = u;
+            for (int e = 0; e < V; ++e) {
+                float a = 0.f;
+#pragma unroll
+                for (int s = 0; s < MAX_STREAMS; ++s)
+                    if (s < S) a = fmaf(w_in[s], x[s][e], a);
+                u[e] = a;
+                ss = fmaf(a, a, ss);
+            }
+            if (norm_w) *(vec*)(us + c) = u;
+            else *(vec*)(u_out + at) = u;
         }
     }
     if (!read || !norm_w) return;
     const float total = block_sum<4>(ss, scratch);
     const float inv = 1.0f / sqrtf(total / (float)d + eps);
-    for (int c = threadIdx.x; c < d; c += 256) h_out[t * d + c] = from_f32<TO>(us[c] * inv * norm_w[c]);
+    for (int c = threadIdx.x * V; c < d; c += 256 * V) {
+        const vec u = *(const vec*)(us + c), w = *(const vec*)(norm_w + c);
+        typedef TO ovec __attribute__((ext_vector_type(V)));
+        ovec o;
+#pragma unroll
+        for (int e = 0; e < V; ++e) o[e] = from_f32<TO>(u[e] * inv * w[e]);
+        *(ovec*)(h_out + t * d + c) = o;
+    }
 }
 }  // namespace
 
@@ -82,11 +111,12 @@ TUFF_EXPORT int tuff_hc_step(float* xs, float* y, const float* mix, const float*
     if ((mix == nullptr) != (out_w == nullptr) || (mix == nullptr) != (y == nullptr)) return -2;
     if (in_w && (norm_w ? h_out == nullptr : u_out == nullptr)) return -2;
     const size_t lds = (size_t)d * sizeof(float);
-    if (out_dt == DT_F32)
-        hipLaunchKernelGGL(hc_step_kernel<float>, dim3(n_tokens), dim3(256), lds, stream, xs, y, mix, out_w, in_w, norm_w,
-                           (float*)h_out, u_out, S, (long long)n_tokens, d, eps, clear_y);
-    else
-        hipLaunchKernelGGL(hc_step_kernel<bf16_t>, dim3(n_tokens), dim3(256), lds, stream, xs, y, mix, out_w, in_w, norm_w,
-                           (bf16_t*)h_out, u_out, S, (long long)n_tokens, d, eps, clear_y);
+    const bool four = d % 4 == 0 && (uintptr_t)xs % 16 == 0 && (!y || (uintptr_t)y % 16 == 0) && (!norm_w || (uintptr_t)norm_w % 16 == 0) &&
+                      (!h_out || (uintptr_t)h_out % 16 == 0) && (!u_out || (uintptr_t)u_out % 16 == 0);
+#define LAUNCH(TO, V) hipLaunchKernelGGL((hc_step_kernel<TO, V>), dim3(n_tokens), dim3(256), lds, stream, xs, y, mix, out_w, in_w, norm_w, \
+                                         (TO*)h_out, u_out, S, (long long)n_tokens, d, eps, clear_y)
+    if (out_dt == DT_F32) { if (four) LAUNCH(float, 4); else LAUNCH(float, 1); }
+    else { if (four) LAUNCH(bf16_t, 4); else LAUNCH(bf16_t, 1); }
+#undef LAUNCH
     return launch_status();
 }
