@@ -11,6 +11,8 @@ a channel's positions contiguous within the page, which is how those kernels rea
 kept once and go through the general kernel.  The expansions are never formed for the
 cached tokens: the query is carried into the latent space, q' = [W_uk,a^T q_plain,a | q_rot,a], attention
 runs over the cache rows as they lie, and W_uv,a is applied to the head's weighted sum of rows.
+Both per-head products (ops.head_matmul) run on the matrix cores in bfloat16 where head sizes, rank and the projected
+row are multiples of 8 (the weights are then also kept with a column's entries together), else in a scalar kernel.
 
 Rotation: neighbouring pairs (2i, 2i + 1) of the first `rot_dims` channels of the rotated part turn by
 position * base^(-2i / rot_dims); the rest passes.
