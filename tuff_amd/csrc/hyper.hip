@@ -22,16 +22,14 @@ __global__ __launch_bounds__(256) void hc_step_kernel(float* __restrict__ xs, fl
                                                       int S, long long T, int d, float eps, int clear_y) {
     extern __shared__ __attribute__((aligned(16))) float us[];     // d floats: the row of u
     __shared__ float scratch[4];
-    __shared__ float w_mix[MAX_STREAMS * MAX_STREAMS], w_out[MAX_STREAMS], w_in[MAX_STREAMS];
     typedef float vec __attribute__((ext_vector_type(V)));
     const long long t = blockIdx.x;
     const bool write = mix != nullptr, read = in_w != nullptr;
-    if (threadIdx.x < S * S && write) w_mix[threadIdx.x] = mix[threadIdx.x];
-    if (threadIdx.x < S) {
-        if (write) w_out[threadIdx.x] = out_w[threadIdx.x];
-        if (read) w_in[threadIdx.x] = in_w[threadIdx.x];
-    }
-    __syncthreads();
+    // the step's few weights are read where they are used: the same address for all lanes, so they come through the
+    // scalar unit beside the row's own loads, and no barrier stands before those
+    const float* __restrict__ w_mix = mix;
+    const float* __restrict__ w_out = out_w;
+    const float* __restrict__ w_in = in_w;
     const long long plane = T * (long long)d;
     float ss = 0.f;
     for (int c = threadIdx.x * V; c < d; c += 256 * V) {
